@@ -3,4 +3,5 @@ from .base import (ConfigError, Architecture, register_architecture, unregister_
 from .llama import LlamaConfig
 from .novosun import NovosunConfig
 from .ditazen import DitazenConfig
+from .noresun import NoresunConfig
 from .presets import preset, preset_names

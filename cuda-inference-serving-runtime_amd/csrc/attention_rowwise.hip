@@ -15,14 +15,16 @@
 #define MAX_HEAD_DIM 640
 #define MAX_COORDS (MAX_HEAD_DIM / WAVE)     // output coordinates a lane
 
-template <typename T>
+// SIGMOID: the weight of a visible key is sigmoid(score + head_bias[head]) and the weights are not normed over the keys
+// (no maximum, no denominator: a row's result is the plain sum, and the partial results of splits are added).
+template <typename T, bool SIGMOID>
 __global__ void __launch_bounds__(64)
 attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restrict__ kcache,
                     const T* __restrict__ vcache, const int* __restrict__ tables,
                     const int* __restrict__ seg_of_row, const int* __restrict__ positions,
                     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
                     int heads, int kv_heads, int dim, int page_size, int width, int window,
-                    float scale, int splits) {
+                    float scale, int splits, const float* __restrict__ head_bias) {
     __shared__ float qs[MAX_HEAD_DIM];
     __shared__ float ps[WAVE];
     __shared__ long long rowoff[WAVE];   // offset of a key's first value element (values are [D, page_size] in a page)
@@ -64,11 +66,19 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
                 for (int d = 0; d < dim; ++d) dot += qs[d] * load_f32(kr + d);
                 s = dot * scale;
             }
-            const float m_new = fmaxf(m, wave_max(s));   // finite: lane 0 of a block is always valid
-            const float pj = valid ? expf(s - m_new) : 0.f;
-            const float alpha = expf(m - m_new);           // exp(-inf) = 0 on the first block
-            l = l * alpha + wave_sum(pj);
-            m = m_new;
+            float pj, alpha;
+            if (SIGMOID) {
+                pj = valid ? 1.0f / (1.0f + expf(-(s + head_bias[head]))) : 0.f;
+                alpha = 1.0f;
+                l = 1.0f;
+                m = 0.f;
+            } else {
+                const float m_new = fmaxf(m, wave_max(s));   // finite: lane 0 of a block is always valid
+                pj = valid ? expf(s - m_new) : 0.f;
+                alpha = expf(m - m_new);           // exp(-inf) = 0 on the first block
+                l = l * alpha + wave_sum(pj);
+                m = m_new;
+            }
             __syncthreads();
             ps[lane] = pj;
             rowoff[lane] = off;
@@ -86,7 +96,7 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
             }
         }
     }
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float inv = SIGMOID ? 1.0f : l > 0.f ? 1.0f / l : 0.f;
     if (splits == 1) {
         T* o = out + ((size_t)row * heads + head) * dim;
 #pragma unroll
@@ -102,6 +112,21 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
             if (c < ncoord && d < dim) part_o[part * dim + d] = acc[c] * inv;
         }
         if (lane == 0) { part_ml[part * 2] = m; part_ml[part * 2 + 1] = l; }
+    }
+}
+
+// Partial results that are plain sums (weights that are not normed over the keys): out = sum_i o_i.
+template <typename T>
+__global__ void attn_merge_sum_kernel(const float* __restrict__ part_o, T* __restrict__ out, int heads, int dim, int splits,
+                                      const int* __restrict__ row_ids = nullptr) {
+    const int head = blockIdx.y;
+    const size_t base = ((size_t)blockIdx.x * heads + head) * splits;
+    const int row = row_ids ? row_ids[blockIdx.x] : (int)blockIdx.x;
+    if (row < 0) return;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float sum = 0.f;
+        for (int s = 0; s < splits; ++s) sum += part_o[(base + s) * dim + d];
+        store_f32(out + ((size_t)row * heads + head) * dim + d, sum);
     }
 }
 
@@ -189,6 +214,40 @@ extern "C" int cisr_attn_merge(const float* part_o, const float* part_ml, void* 
     return CISR_LAUNCH_CHECK();
 }
 
+// merge of the matrix-core kernel's partials where they are plain sums (bf16 output)
+extern "C" int cisr_attn_merge_sum(const float* part_o, void* out, int rows, int heads, int dim, int splits, const int* row_ids,
+                                   hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (heads > 65535 || splits < 1) return (int)hipErrorInvalidValue;
+    attn_merge_sum_kernel<bf16_t><<<dim3(rows, heads), merge_threads(dim), 0, stream>>>(part_o, (bf16_t*)out, heads, dim, splits, row_ids);
+    return CISR_LAUNCH_CHECK();
+}
+
+// The same attention with weights sigmoid(score + head_bias[head]) that are not normed over the keys.
+extern "C" int cisr_attn_rowwise_sigmoid(const void* q, int q_row_stride, const void* kcache, const void* vcache,
+                                         const int* tables, const int* seg_of_row, const int* positions, void* out,
+                                         float* part_o, float* part_ml, int rows, int heads, int kv_heads, int dim,
+                                         int page_size, int width, int window, float scale, int splits, int dtype,
+                                         const float* head_bias, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim > MAX_HEAD_DIM || dim <= 0 || heads % kv_heads || splits < 1 || splits > 65535 || heads > 65535 || !head_bias)
+        return (int)hipErrorInvalidValue;
+    dim3 grid(rows, heads, splits);
+    if (dtype == DT_F32)
+        attn_rowwise_kernel<float, true><<<grid, 64, 0, stream>>>((const float*)q, q_row_stride, (const float*)kcache,
+            (const float*)vcache, tables, seg_of_row, positions, (float*)out, part_o, part_ml, heads, kv_heads,
+            dim, page_size, width, window, scale, splits, head_bias);
+    else
+        attn_rowwise_kernel<bf16_t, true><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_row_stride, (const bf16_t*)kcache,
+            (const bf16_t*)vcache, tables, seg_of_row, positions, (bf16_t*)out, part_o, part_ml, heads, kv_heads,
+            dim, page_size, width, window, scale, splits, head_bias);
+    int err = CISR_LAUNCH_CHECK();
+    if (err || splits == 1) return err;
+    if (dtype == DT_F32) attn_merge_sum_kernel<float><<<dim3(rows, heads), merge_threads(dim), 0, stream>>>(part_o, (float*)out, heads, dim, splits);
+    else attn_merge_sum_kernel<bf16_t><<<dim3(rows, heads), merge_threads(dim), 0, stream>>>(part_o, (bf16_t*)out, heads, dim, splits);
+    return CISR_LAUNCH_CHECK();
+}
+
 extern "C" int cisr_attn_rowwise(const void* q, int q_row_stride, const void* kcache, const void* vcache,
                                  const int* tables, const int* seg_of_row, const int* positions, void* out,
                                  float* part_o, float* part_ml, int rows, int heads, int kv_heads, int dim,
@@ -199,13 +258,13 @@ extern "C" int cisr_attn_rowwise(const void* q, int q_row_stride, const void* kc
         return (int)hipErrorInvalidValue;
     dim3 grid(rows, heads, splits);
     if (dtype == DT_F32)
-        attn_rowwise_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_row_stride, (const float*)kcache,
+        attn_rowwise_kernel<float, false><<<grid, 64, 0, stream>>>((const float*)q, q_row_stride, (const float*)kcache,
             (const float*)vcache, tables, seg_of_row, positions, (float*)out, part_o, part_ml, heads, kv_heads,
-            dim, page_size, width, window, scale, splits);
+            dim, page_size, width, window, scale, splits, nullptr);
     else
-        attn_rowwise_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_row_stride, (const bf16_t*)kcache,
+        attn_rowwise_kernel<bf16_t, false><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_row_stride, (const bf16_t*)kcache,
             (const bf16_t*)vcache, tables, seg_of_row, positions, (bf16_t*)out, part_o, part_ml, heads, kv_heads,
-            dim, page_size, width, window, scale, splits);
+            dim, page_size, width, window, scale, splits, nullptr);
     int err = CISR_LAUNCH_CHECK();
     if (err || splits == 1) return err;
     const int threads = merge_threads(dim);

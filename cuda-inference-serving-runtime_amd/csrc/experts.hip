@@ -1,0 +1,282 @@
+// Routed experts: each row of a step goes through the `top` experts with the largest router logits.
+//
+//   route      logits float [T, E] (+ bias) -> the chosen experts [T, top] (largest first, the lowest index wins a tie)
+//              and their weights, the softmax over the chosen logits only, float
+//   arrange    the T top (row, choice) pairs ordered by expert, every expert's run padded to a whole number of 64-row
+//              tiles: pair_of_pos[pos] (-1: padding) and tile_expert[tile] (-1: no tile).  One block; the order of
+//              pairs inside an expert's run is whatever the atomics give, which no result depends on (a pair's
+//              arithmetic does not know its place).
+//   products   per tile of 64 pairs one expert's matrix: up  = act(h[row of pair] . Wup[e]^T) stored by place,
+//              down = up[place] . Wdown[e]^T stored by pair, float [T top, H]; the weighted sum over a row's pairs
+//              is left to the kernel that reads them next.
+// bf16 operands run on the matrix cores (K a multiple of 8, 16-byte aligned rows); everything else, and the true
+// 32-bit path, runs the plain FMA kernel with float accumulation in ascending k order.
+#include "common.h"
+
+#define EX_TILE 64
+#define MAX_TOP 16
+
+__global__ void __launch_bounds__(256)
+route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias, int* __restrict__ chosen,
+             float* __restrict__ weights, int rows, int experts, int top) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= rows) return;
+    const float* lr = logits + (size_t)row * ld;
+    int ids[MAX_TOP];
+    float vals[MAX_TOP];
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bv = -INFINITY;
+        for (int e = 0; e < experts; ++e) {
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= ids[j] == e;
+            if (taken) continue;
+            const float v = lr[e] + (bias ? bias[e] : 0.f);
+            if (best < 0 || v > bv) { best = e; bv = v; }
+        }
+        ids[k] = best;
+        vals[k] = bv;
+    }
+    float den = 0.f;
+    const float largest = vals[0];
+    for (int k = 0; k < top; ++k) { vals[k] = expf(vals[k] - largest); den += vals[k]; }
+    for (int k = 0; k < top; ++k) {
+        chosen[(size_t)row * top + k] = ids[k];
+        weights[(size_t)row * top + k] = vals[k] / den;
+    }
+}
+
+__global__ void __launch_bounds__(1024)
+arrange_kernel(const int* __restrict__ chosen, int pairs, int experts, int max_tiles, int* __restrict__ pair_of_pos,
+               int* __restrict__ tile_expert) {
+    extern __shared__ int lds[];          // counts[E], then start[E] (in places), then cursor[E]
+    int* counts = lds;
+    int* start = lds + experts;
+    int* cursor = lds + 2 * experts;
+    for (int e = threadIdx.x; e < experts; e += 1024) counts[e] = 0;
+    for (int p = threadIdx.x; p < max_tiles * EX_TILE; p += 1024) pair_of_pos[p] = -1;
+    for (int t = threadIdx.x; t < max_tiles; t += 1024) tile_expert[t] = -1;
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += 1024) {
+        const int e = chosen[p];
+        if (e >= 0 && e < experts) atomicAdd(&counts[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int e = 0; e < experts; ++e) {
+            start[e] = cursor[e] = at;
+            at += (counts[e] + EX_TILE - 1) / EX_TILE * EX_TILE;
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += 1024) {
+        const int first = start[e] / EX_TILE, n = (counts[e] + EX_TILE - 1) / EX_TILE;
+        for (int t = 0; t < n; ++t) if (first + t < max_tiles) tile_expert[first + t] = e;
+    }
+    for (int p = threadIdx.x; p < pairs; p += 1024) {
+        const int e = chosen[p];
+        if (e < 0 || e >= experts) continue;
+        const int pos = atomicAdd(&cursor[e], 1);
+        if (pos < max_tiles * EX_TILE) pair_of_pos[pos] = p;
+    }
+}
+
+extern "C" int cisr_experts_route(const float* logits, int ld, const float* bias, int* chosen, float* weights, int rows,
+                                  int experts, int top, int max_tiles, int* pair_of_pos, int* tile_expert, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (experts <= 0 || top <= 0 || top > MAX_TOP || top > experts || experts > 4096 ||
+        (long long)max_tiles * EX_TILE < (long long)rows * top + (long long)experts * (EX_TILE - 1))
+        return (int)hipErrorInvalidValue;
+    route_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(logits, ld, bias, chosen, weights, rows, experts, top);
+    int err = CISR_LAUNCH_CHECK();
+    if (err) return err;
+    arrange_kernel<<<1, 1024, 3 * experts * sizeof(int), stream>>>(chosen, rows * top, experts, max_tiles, pair_of_pos, tile_expert);
+    return CISR_LAUNCH_CHECK();
+}
+
+// relu(z)^2, the experts' activation; ACT 0: none
+template <int ACT>
+__device__ __forceinline__ float expert_act(float v) {
+    if (ACT == 0) return v;
+    const float r = fmaxf(v, 0.f);
+    return r * r;
+}
+
+// rows of a tile: where the operand's row of a place lies, and where its result goes (-1: padding)
+struct TileRows { int a, c; };
+__device__ __forceinline__ TileRows tile_rows(int pos, int pair, int gather_div, int scatter) {
+    TileRows t;
+    t.a = pair < 0 ? -1 : gather_div > 0 ? pair / gather_div : pos;
+    t.c = pair < 0 ? -1 : scatter ? pair : pos;
+    return t;
+}
+
+// ------------------------------------------------------------------ plain FMA tiles (any type, any size)
+template <typename TA, typename TC, int ACT>
+__global__ void __launch_bounds__(256)
+expert_gemm_fma_kernel(const TA* __restrict__ A, int lda, const TA* __restrict__ W, const int* __restrict__ tile_expert,
+                       const int* __restrict__ pair_of_pos, int gather_div, int scatter, TC* __restrict__ C, int ldc, int N, int K) {
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    __shared__ float As[16][EX_TILE + 4];
+    __shared__ float Ws[16][EX_TILE + 4];
+    __shared__ int arow[EX_TILE], crow[EX_TILE];
+    const int tid = threadIdx.x;
+    if (tid < EX_TILE) {
+        const int pos = tile * EX_TILE + tid;
+        const TileRows t = tile_rows(pos, pair_of_pos[pos], gather_div, scatter);
+        arow[tid] = t.a; crow[tid] = t.c;
+    }
+    __syncthreads();
+    const int n0 = blockIdx.y * EX_TILE;
+    const TA* We = W + (size_t)e * N * K;
+    const int ty = tid / 16, tx = tid % 16;
+    const int lr = tid / 4, lk = (tid % 4) * 4;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int k = k0 + lk + x;
+            const int am = arow[lr], wn = n0 + lr;
+            As[lk + x][lr] = (am >= 0 && k < K) ? load_f32(A + (size_t)am * lda + k) : 0.f;
+            Ws[lk + x][lr] = (wn < N && k < K) ? load_f32(We + (size_t)wn * K + k) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = crow[ty * 4 + i];
+        if (m < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) store_f32(C + (size_t)m * ldc + n, expert_act<ACT>(acc[i][j]));
+        }
+    }
+}
+
+// ------------------------------------------------------------------ matrix-core tiles (bf16, K a multiple of 8)
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+#define EX_BK 32
+#define EX_LD 40         // bf16 elements a tile row takes in LDS (80 bytes: 16-byte chunks, rows spread over the banks)
+
+// A block of four waves owns 64 places x 64 columns; wave w the places 16 w .. 16 w + 15 and all four column tiles.
+// Operands go global memory -> registers -> LDS (two buffers, one barrier a 32-deep step) -> matrix-core operands.
+template <typename TC, int ACT>
+__global__ void __launch_bounds__(256)
+expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const int* __restrict__ tile_expert,
+                        const int* __restrict__ pair_of_pos, int gather_div, int scatter, TC* __restrict__ C, int ldc, int N, int K) {
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][EX_TILE * EX_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][EX_TILE * EX_LD];
+    __shared__ int crow[EX_TILE];
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int lr = tid / 4, lc = (tid % 4) * 8;               // this thread's chunk of a tile: row, first k
+    const int n0 = blockIdx.y * EX_TILE;
+    const int pos = tile * EX_TILE + lr;
+    const TileRows mine = tile_rows(pos, pair_of_pos[pos], gather_div, scatter);
+    if (tid % 4 == 0) crow[lr] = mine.c;
+    const bf16_t* ap = mine.a >= 0 ? A + (size_t)mine.a * lda : nullptr;
+    const bf16_t* wp = n0 + lr < N ? W + ((size_t)e * N + n0 + lr) * K : nullptr;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    auto fetch = [&](int k0, u32x4& va, u32x4& vw) {
+        const int k = k0 + lc;
+        va = (ap && k < K) ? *(const u32x4*)(ap + k) : zero;
+        vw = (wp && k < K) ? *(const u32x4*)(wp + k) : zero;
+    };
+    f32x4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    u32x4 va, vw;
+    fetch(0, va, vw);
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += EX_BK) {
+        *(u32x4*)(&As[buf][lr * EX_LD + lc]) = va;
+        *(u32x4*)(&Ws[buf][lr * EX_LD + lc]) = vw;
+        __syncthreads();       // whoever writes this buffer again, two steps on, has passed the next step's barrier
+        if (k0 + EX_BK < K) fetch(k0 + EX_BK, va, vw);
+        const bf16x8 fa = *(const bf16x8*)(&As[buf][(wave * 16 + r) * EX_LD + g * 8]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bf16x8 fw = *(const bf16x8*)(&Ws[buf][(j * 16 + r) * EX_LD + g * 8]);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fw, acc[j], 0, 0, 0);
+        }
+        buf ^= 1;
+    }
+    // a lane holds rows 4 g .. 4 g + 3 of column r in every 16 x 16 tile
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        const int m = crow[wave * 16 + g * 4 + x];
+        if (m < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + j * 16 + r;
+            if (n < N) store_f32(C + (size_t)m * ldc + n, expert_act<ACT>(acc[j][x]));
+        }
+    }
+}
+
+// C[c row of place] = act(A[a row of place] . W[expert of the place's tile]^T); W is [experts, N, K].
+// gather_div > 0: the operand's row of a place is pair / gather_div (a step's row), else the place itself;
+// scatter: the result goes to row `pair`, else to the place.  dtype: of A and W; out_dtype: of C.
+extern "C" int cisr_experts_gemm(const void* A, int lda, const void* W, const int* tile_expert, const int* pair_of_pos,
+                                 int gather_div, int scatter, void* C, int ldc, int max_tiles, int N, int K, int act,
+                                 int dtype, int out_dtype, hipStream_t stream) {
+    if (max_tiles <= 0 || N <= 0) return 0;
+    if (K <= 0 || max_tiles > 0x7fffff || (N + EX_TILE - 1) / EX_TILE > 65535 || (dtype == DT_F32 && out_dtype != DT_F32))
+        return (int)hipErrorInvalidValue;
+    const dim3 grid(max_tiles, (N + EX_TILE - 1) / EX_TILE);
+#define EX_ARGS tile_expert, pair_of_pos, gather_div, scatter
+    if (dtype == DT_F32) {
+        if (act) expert_gemm_fma_kernel<float, float, 1><<<grid, 256, 0, stream>>>((const float*)A, lda, (const float*)W, EX_ARGS, (float*)C, ldc, N, K);
+        else expert_gemm_fma_kernel<float, float, 0><<<grid, 256, 0, stream>>>((const float*)A, lda, (const float*)W, EX_ARGS, (float*)C, ldc, N, K);
+        return CISR_LAUNCH_CHECK();
+    }
+    const bool vec = K % 8 == 0 && lda % 8 == 0 && ((uintptr_t)A) % 16 == 0 && ((uintptr_t)W) % 16 == 0;
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    if (vec) {
+        if (out_dtype == DT_F32) {
+            if (act) expert_gemm_mfma_kernel<float, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+            else expert_gemm_mfma_kernel<float, 0><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+        } else {
+            if (act) expert_gemm_mfma_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+            else expert_gemm_mfma_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+        }
+    } else {
+        if (out_dtype == DT_F32) {
+            if (act) expert_gemm_fma_kernel<bf16_t, float, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+            else expert_gemm_fma_kernel<bf16_t, float, 0><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+        } else {
+            if (act) expert_gemm_fma_kernel<bf16_t, bf16_t, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+            else expert_gemm_fma_kernel<bf16_t, bf16_t, 0><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+        }
+    }
+#undef EX_ARGS
+    return CISR_LAUNCH_CHECK();
+}

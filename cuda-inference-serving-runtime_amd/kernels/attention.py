@@ -291,11 +291,12 @@ def fused_merge_splits(splits, rows, accepts):
 
 # -- the call ---------------------------------------------------------------------------------------------------
 
-def kernel_units(head_dim, dtype):
-    """Names of the shared objects that attention with this head size needs beside the core (library.ensure)."""
+def kernel_units(head_dim, dtype, law="softmax"):
+    """Names of the shared objects that attention with this head size needs beside the core (library.ensure).
+    `law` "sigmoid": the build with sigmoid weights that are not normed over the keys."""
     from . import library
     if dtype == torch.bfloat16 and head_dim % 8 == 0 and 0 < head_dim <= 256:
-        return [library.attention_unit(-(-head_dim // 32) * 32)]
+        return [library.attention_unit(-(-head_dim // 32) * 32, law)]
     return []
 
 
@@ -305,10 +306,14 @@ def _split_workspace(ctx, rows, heads, splits, head_dim, dtype=torch.float32, ta
 
 
 def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale,
-                    defer_merge=None, tuning=DEFAULT_TUNING):
+                    defer_merge=None, tuning=DEFAULT_TUNING, head_bias=None):
     """out[r] = attention of row r's queries over its request's cached keys up to its own position (or the last
     `window` of them).  `ctx` is the step's context (rows, segments, positions, buffers, step arrays), `view` the
     cache group as the step sees it (block tables, page size).
+
+    `head_bias` (float [heads]): the sigmoid law: a visible key weighs sigmoid(score + head_bias[head]) and the weights
+    are not normed over the keys.  Same kernels, launch rules and step arrays, except that prompt rows always run as
+    tiles (the forms through LDS have no such build) and no later product merges split keys.
 
     `defer_merge(splits) -> bool`: the caller's next product can merge the partial results of a decode step whose
     keys are split over `splits` blocks itself (ops.gemm_merged).  Where that is so, no merge kernel runs, `out`
@@ -320,7 +325,7 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
     if not ops.mfma_attention_supported(out.dtype, head_dim, view.page_size):
         splits = rowwise_splits(rows * heads, span)
         workspace = _split_workspace(ctx, rows, heads, splits, head_dim) if splits > 1 else None
-        ops.attention_rowwise(*common, splits, workspace)
+        ops.attention_rowwise(*common, splits, workspace, head_bias=head_bias)
         return None
     group = heads // kv_heads
     heads_per_chunk = min(group, 16)
@@ -333,7 +338,7 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
 
     if ctx.decode_only:
         waves, splits = tuning.rows_launch or rows_launch(rows * chunks, span, heads_per_chunk, head_dim)
-        if splits > 1 and defer_merge is not None:
+        if splits > 1 and defer_merge is not None and head_bias is None:
             fused = fused_merge_splits(splits, rows, defer_merge)
             if fused is not None:
                 workspace = _split_workspace(ctx, rows, heads, fused, head_dim, torch.bfloat16, "attn.part_o16")
@@ -344,7 +349,8 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
         order = None
         if splits == 1 and rows * chunks >= tuning.order_rows_from:
             order = ctx.step_array(RowsLongestFirst())[0][:rows]
-        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=order, stream_loads=stream(rows * chunks, waves, splits))
+        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=order, stream_loads=stream(rows * chunks, waves, splits),
+                           head_bias=head_bias)
         return None
     singles = SingleRows(tuning.split_single_from)
     single_rows, n_single = ctx.step_array(singles)
@@ -353,10 +359,13 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
         waves, splits = tuning.rows_launch or rows_launch(n_single * chunks, span, heads_per_chunk, head_dim)
         workspace = _split_workspace(ctx, n_single, heads, splits, head_dim) if splits > 1 else None
         ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=single_rows[:n_single],
-                           stream_loads=stream(n_single * chunks, waves, splits))
+                           stream_loads=stream(n_single * chunks, waves, splits), head_bias=head_bias)
     form = prompt_form(rows, ctx.n_segments, span, heads, kv_heads, head_dim, view.page_size, tuning)
+    if head_bias is not None and form[0] != "tiles":
+        form = ("tiles", 2 if tuning.item_tiles == 2 and head_dim <= 64 else 1, 1)
     kind, item_tiles, halves = form
     tasks, _ = ctx.step_array(TileTasks(rows_per_tile_of(form, heads, kv_heads), singles))
     ops.attention_mfma(*common, tasks.view(-1, 4), waves=tuning.tile_waves,
-                       block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles, key_groups=halves)
+                       block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles, key_groups=halves,
+                       head_bias=head_bias)
     return None

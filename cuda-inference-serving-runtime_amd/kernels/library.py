@@ -49,19 +49,21 @@ def _log(msg):
     print(f"[runtime.kernels] {msg}", file=sys.stderr, flush=True)
 
 
-def attention_unit(dpad):
-    return f"attn_d{dpad}"
+def attention_unit(dpad, law="softmax"):
+    """The unit of the matrix-core attention of a padded head size; `law` "sigmoid": weights sigmoid(score + a bias a
+    head) that are not normed over the keys."""
+    return f"attn_sig_d{dpad}" if law == "sigmoid" else f"attn_d{dpad}"
 
 
 def units():
     """The shared objects the kernels are built into: the core, and one per padded head size of the
     matrix-core attention (a model needs only its own, so a first call compiles only that one)."""
-    return [CORE, *OWN_UNITS] + [attention_unit(d) for d in ATTENTION_PADS]
+    return [CORE, *OWN_UNITS] + [attention_unit(d, law) for law in ("softmax", "sigmoid") for d in ATTENTION_PADS]
 
 
 def sources(unit=CORE):
     if unit == CORE:
-        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d") and not p.stem.startswith(OWN_UNITS))
+        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_") and not p.stem.startswith(OWN_UNITS))
     if unit in OWN_UNITS:
         return sorted(CSRC.glob(f"{unit}*.hip"))
     path = CSRC / f"attention_mfma_{unit[len('attn_'):]}.hip"
@@ -183,10 +185,10 @@ def load(unit=CORE):
         return handle
 
 
-def load_attention(dpad):
+def load_attention(dpad, law="softmax"):
     if dpad not in ATTENTION_PADS:
         raise KernelLibraryError(f"no matrix-core attention for a padded head size of {dpad}")
-    return load(attention_unit(dpad))
+    return load(attention_unit(dpad, law))
 
 
 def loaded_path(unit=CORE):

@@ -81,6 +81,13 @@ def _declare(h):
         "cisr_gemm_bf16_heads": [p, i, i, p, p, i, i, p, i, i, i, i, i, i, p],
         "cisr_gemm_skinny_bf16_act": [p, i, p, i, p, i, i, i, i, i, i, p],
         "cisr_gemm_bf16_act": [p, i, p, i, p, i, i, i, i, i, i, p],
+        "cisr_attn_rowwise_sigmoid": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p, p],
+        "cisr_attn_merge_sum": [p, p, i, i, i, i, p, p],
+        "cisr_embedding_pairs": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, f, i, ll, ll, i, i, i, p],
+        "cisr_gate_post_norm": [p, p, i, p, p, i, p, p, p, i, i, f, f, i, p],
+        "cisr_whole_norm_rope_scatter": [p, i, p, p, p, p, p, p, i, i, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
+        "cisr_experts_route": [p, i, p, p, p, i, i, i, i, p, p, p],
+        "cisr_experts_gemm": [p, i, p, p, p, i, i, p, i, i, i, i, i, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -97,16 +104,18 @@ def _declare(h):
 _attention_entries = {}
 
 
-def _attention_entry(dpad):
+def _attention_entry(dpad, law="softmax"):
     """The matrix-core attention entry point for a padded head size (its shared object is built and loaded
-    at the first use of that size)."""
-    fn = _attention_entries.get(dpad)
+    at the first use of that size).  `law` "sigmoid": the build whose weights are sigmoid(score + a bias a head), not
+    normed over the keys; its entry takes the biases as a last argument."""
+    fn = _attention_entries.get((dpad, law))
     if fn is None:
         p, i, f = C.c_void_p, C.c_int, C.c_float
-        fn = getattr(library.load_attention(dpad), f"cisr_attn_mfma_d{dpad}")
-        fn.argtypes = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, i, p]
+        sigmoid = law == "sigmoid"
+        fn = getattr(library.load_attention(dpad, law), f"cisr_attn_mfma_sig_d{dpad}" if sigmoid else f"cisr_attn_mfma_d{dpad}")
+        fn.argtypes = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, i, p] + ([p] if sigmoid else [])
         fn.restype = C.c_int
-        _attention_entries[dpad] = fn
+        _attention_entries[(dpad, law)] = fn
     return fn
 
 
@@ -304,9 +313,11 @@ ROWWISE_MAX_HEAD = 640     # the row-wise attention kernel's largest head (the m
 
 
 def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
-                      page_size, window, scale, splits=1, workspace=None):
+                      page_size, window, scale, splits=1, workspace=None, head_bias=None):
     """Each row attends to its request's cached keys lo..position.  q is a view
-    into a row-major buffer with `q_row_stride` elements per row; out [T, heads*dim]."""
+    into a row-major buffer with `q_row_stride` elements per row; out [T, heads*dim].
+    `head_bias` (float [heads]): the weight of a visible key is sigmoid(score + head_bias[head]) instead of its share
+    of a softmax, and the weights are not normed over the keys."""
     rows = out.shape[0]
     dt = _storage(out, "out")
     if dim % 2 or dim > ROWWISE_MAX_HEAD:
@@ -328,12 +339,15 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
         pm = _dev(part_ml, "part_ml", torch.float32)
         if part_o.numel() < rows * heads * splits * dim or part_ml.numel() < rows * heads * splits * 2:
             raise KernelError("attention: split workspace too small")
-    _check(lib().cisr_attn_rowwise(q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
-                                   _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)),
-                                   _dev(tables, "tables", torch.int32), _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
-                                   _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)),
-                                   po, pm, rows, heads, kv_heads, dim, page_size, width, int(window or 0), float(scale),
-                                   int(splits), dt, _stream()), "attention_rowwise")
+    args = (q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
+            _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)),
+            _dev(tables, "tables", torch.int32), _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
+            _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)),
+            po, pm, rows, heads, kv_heads, dim, page_size, width, int(window or 0), float(scale), int(splits), dt)
+    if head_bias is not None:
+        _check(lib().cisr_attn_rowwise_sigmoid(*args, _dev(head_bias, "head_bias", torch.float32, (heads,)), _stream()), "attention_rowwise")
+    else:
+        _check(lib().cisr_attn_rowwise(*args, _stream()), "attention_rowwise")
     return out
 
 
@@ -718,7 +732,7 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                    page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False,
-                   item_tiles=1, row_ids=None, merge=True, key_groups=1, stream_loads=False):
+                   item_tiles=1, row_ids=None, merge=True, key_groups=1, stream_loads=False, head_bias=None):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
     prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
     64: 32/GC rows, two item tiles a wave), or with `block_tiles` (head sizes up to 128) one tile of
@@ -730,8 +744,12 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     `merge` False (rows mode with splits > 1): the partial outputs are left unmerged in the workspace, whose first
     buffer is then bfloat16, for gemm_merged; `out` is not written.  `key_groups` 2 (block_tiles 32): a block is two
     halves that take the even and the odd 32-key steps of its items and merge at the end.  `stream_loads` (rows mode):
-    keys and values are read with non-temporal loads, which the caches do not keep."""
+    keys and values are read with non-temporal loads, which the caches do not keep.
+    `head_bias` (float [heads]): the sigmoid law (see attention_rowwise); the tile and row forms have it, the block
+    tiles do not, and the partial results of split keys are plain sums that only this function merges."""
     rows = out.shape[0]
+    if head_bias is not None and (block_tiles or not merge):
+        raise KernelError("attention_mfma: the sigmoid law runs as tiles and rows, merged here")
     if not mfma_attention_supported(out.dtype, dim, page_size):
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
     if heads % kv_heads:
@@ -746,7 +764,8 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     if kcache.numel() >= 2 ** 31 or vcache.numel() >= 2 ** 31:
         raise KernelError("attention_mfma: a layer's keys (or values) must be fewer than 2^31 elements (32-bit byte offsets)")
     dpad = -(-dim // 32) * 32
-    fn = _attention_entry(dpad)
+    fn = _attention_entry(dpad, "softmax" if head_bias is None else "sigmoid")
+    law = () if head_bias is None else (_dev(head_bias, "head_bias", torch.float32, (heads,)),)
     po = pm = tp = None
     if tasks is not None:
         if item_tiles not in ((1, 2, 3, 4) if block_tiles == 32 else (1, 2)) or (item_tiles == 2 and dim > 64 and not block_tiles):
@@ -785,9 +804,12 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
               _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)), po, pm,
               heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits),
               11 if mode == 1 and stream_loads else mode, int(waves),
-              int(mode == 1 and splits > 1 and not merge), _stream()), "attention_mfma")
+              int(mode == 1 and splits > 1 and not merge), _stream(), *law), "attention_mfma")
     if mode == 1 and splits > 1 and merge:
-        _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), n_tasks, heads, dim, int(splits), tp, _stream()), "attention_merge")
+        if head_bias is not None:
+            _check(lib().cisr_attn_merge_sum(po, out.data_ptr(), n_tasks, heads, dim, int(splits), tp, _stream()), "attention_merge")
+        else:
+            _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), n_tasks, heads, dim, int(splits), tp, _stream()), "attention_merge")
     return out
 
 
@@ -1105,6 +1127,7 @@ def _rec():
             "cisr_group_norm_gate": [p, p, i, p, i, p, i, p, i, p, i, i, i, f, i, i, p],
             "cisr_delta_scan": [p, i, p, i, p, i, p, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
             "cisr_unit_heads": [p, i, i, i, i, i, f, f, p],
+            "cisr_mingru_scan": [p, i, p, p, p, i, p, p, p, i, i, i, i, p, i, i, p],
         }
         for name, args in sig.items():
             fn = getattr(h, name)
@@ -1316,4 +1339,186 @@ def delta_scan(q, k, v, decay, write, out, state, seg_start, state_slots, heads,
                                   _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, R, Cc,
                                   int(share), float(q_scale), cols, _stream()), "delta_scan")
+    return out
+
+
+# -- layers that norm after the sum, hashed token pairs, whole-projection norms (csrc/elementwise_postnorm.hip) --------
+
+def embedding_pairs(tokens, positions, seg_of_row, seg_start, state_slots, table, out, scale=1.0, pairs=None, last_token=None,
+                    buckets=0, mul_prev=0, mul_cur=0, cast=None, single_rows=False):
+    """out[r] = table[tokens[r]] * scale (+ pairs[(previous token * mul_prev + token * mul_cur) mod buckets], or row
+    `buckets` of `pairs` at position 0), float [T, H].  The token before a segment's first row is last_token[state slot]
+    (int32 [slots]), which afterwards holds the segment's last token.  `cast`: a copy of the rows in the table's type.
+    `single_rows`: every segment brings one row (one launch instead of two)."""
+    rows = tokens.shape[0]
+    vocab, dim = table.shape
+    segments = state_slots.shape[0]
+    pp = lp = None
+    if pairs is not None:
+        if last_token is None or buckets <= 0 or pairs.dtype != table.dtype:
+            raise KernelError("embedding_pairs: the pair table needs its buckets, the kept tokens and the table's dtype")
+        pp = _dev(pairs, "pairs", None, (buckets + 1, dim))
+        lp = _dev(last_token, "last_token", torch.int32)
+        if last_token.numel() < 1:
+            raise KernelError("embedding_pairs: no kept tokens")
+    cp, cdt = None, _storage(table, "table")
+    if cast is not None:
+        cp, cdt = _dev(cast, "cast", None, (rows, dim)), _storage(cast, "cast")
+        if cast.dtype != table.dtype:
+            raise KernelError("embedding_pairs: the copy has the table's dtype")
+    _check(lib().cisr_embedding_pairs(_dev(tokens, "tokens", torch.int32, (rows,)), _dev(positions, "positions", torch.int32, (rows,)),
+                                      _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
+                                      _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
+                                      _dev(state_slots, "state_slots", torch.int32, (segments,)), lp, _dev(table, "table"), pp,
+                                      _dev(out, "out", torch.float32, (rows, dim)), cp, rows, segments, dim, vocab, float(scale),
+                                      int(buckets), int(mul_prev), int(mul_cur), int(bool(single_rows)), _storage(table, "table"), cdt,
+                                      _stream()), "embedding_pairs")
+    return out
+
+
+class WeightedRows:
+    """A sublayer's result as `top` rows a step row, to be summed with weights by the kernel that reads it next
+    (gate_post_norm): rows float [T * top, H], weights float [T, top]."""
+
+    def __init__(self, rows, weights, top):
+        self.rows, self.weights, self.top = rows, weights, int(top)
+
+
+def gate_post_norm(x, y, weight, eps, alpha, gate=None, gate_bias=None, cast=None):
+    """x <- rmsnorm(alpha x + y * sigmoid(gate + gate_bias)) * weight, in place (float [T, H]); y float [T, H] or a
+    WeightedRows; `gate` a float view [T, H] with unit column stride (None: no gate); `cast` [T, H]: a copy of the
+    new rows in the activations' type."""
+    rows, dim = x.shape
+    top, yw = 1, None
+    if isinstance(y, WeightedRows):
+        top = y.top
+        yp = _dev(y.rows, "y", torch.float32, (rows * top, dim))
+        yw = _dev(y.weights, "y weights", torch.float32, (rows, top))
+    else:
+        yp = _dev(y, "y", torch.float32, (rows, dim))
+    gp, ldg, gb = None, 0, None
+    if gate is not None:
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (rows, dim) or gate.stride(1) != 1 or not gate.is_cuda:
+            raise KernelError("gate_post_norm: the gate is a float view [T, H] with unit column stride")
+        gp, ldg = gate.data_ptr(), gate.stride(0)
+        gb = None if gate_bias is None else _dev(gate_bias, "gate_bias", torch.float32, (dim,))
+    cp, cdt = None, F32
+    if cast is not None:
+        cp, cdt = _dev(cast, "cast", None, (rows, dim)), _storage(cast, "cast")
+    _check(lib().cisr_gate_post_norm(_dev(x, "x", torch.float32), yp, top, yw, gp, ldg, gb, _dev(weight, "weight", torch.float32, (dim,)),
+                                     cp, rows, dim, float(eps), float(alpha), cdt, _stream()), "gate_post_norm")
+    return x
+
+
+def whole_norm_rope_scatter(proj, q_norm, k_norm, positions, slots, cos, sin, q_out, kcache, vcache, heads, kv_heads, dim, vdim,
+                            pad, page_size, eps):
+    """Rows of a projection with float results [q: heads x dim | k: kv_heads x dim | v: kv_heads x vdim | ...]: q and k
+    RMS-normed over all their heads at once (weights float [heads * dim], [kv_heads * dim]), the first 2 * cos.shape[1]
+    coordinates of every head turned in neighbouring pairs by the position (cos / sin float [max_pos, pairs]), q into
+    q_out [T, heads * pad], k and v into the pages at `slots` as heads of `pad` coordinates whose rest is zero.
+    kcache None: the rows have queries only (a layer that reads another's cache)."""
+    rows, ld = proj.shape
+    has_kv = kcache is not None
+    if proj.dtype != torch.float32 or proj.stride(1) != 1 or not proj.is_cuda:
+        raise KernelError("whole_norm_rope_scatter: a float projection with contiguous rows")
+    if dim > pad or vdim > pad or ld < heads * dim + (kv_heads * (dim + vdim) if has_kv else 0):
+        raise KernelError(f"whole_norm_rope_scatter: heads of {dim} / {vdim} do not fit rows of {ld} or pages of {pad}")
+    max_pos, half = cos.shape
+    if 2 * half > dim:
+        raise KernelError(f"whole_norm_rope_scatter: {2 * half} turning coordinates in heads of {dim}")
+    kp = vp = sp = kw = None
+    if has_kv:
+        pages = kcache.shape[0]
+        kp = _dev(kcache, "kcache", q_out.dtype, (pages, kv_heads, page_size, pad))
+        vp = _dev(vcache, "vcache", q_out.dtype, (pages, kv_heads, pad, page_size))
+        sp = _dev(slots, "slots", torch.int32, (rows,))
+        kw = _dev(k_norm, "k_norm", torch.float32, (kv_heads * dim,))
+    _check(lib().cisr_whole_norm_rope_scatter(proj.data_ptr(), proj.stride(0), _dev(q_norm, "q_norm", torch.float32, (heads * dim,)), kw,
+                                              _dev(positions, "positions", torch.int32, (rows,)), sp,
+                                              _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, half)),
+                                              half, max_pos, _dev(q_out, "q_out", None, (rows, heads * pad)), kp, vp, rows, heads,
+                                              kv_heads, dim, vdim, pad, page_size, float(eps), int(has_kv), _storage(q_out, "q_out"),
+                                              _stream()), "whole_norm_rope_scatter")
+    return q_out
+
+
+# -- routed experts (csrc/experts.hip) -----------------------------------------------------------------------------
+
+EXPERT_TILE = 64      # rows of a tile of the experts' products: every expert's rows are padded to a multiple
+
+
+def expert_tiles(rows, top, experts):
+    """Tiles that the rows of a step can take at most once ordered by expert (every expert's run padded to whole tiles)."""
+    return -(-rows * top // EXPERT_TILE) + experts
+
+
+def experts_route(logits, bias, top, chosen, weights, pair_of_pos, tile_expert):
+    """logits: a float view [T, E] with unit column stride (+ bias float [E]) -> chosen int32 [T, top] (largest first,
+    the lowest index wins a tie), weights float [T, top] (softmax over the chosen logits), and the (row, choice) pairs
+    ordered by expert: pair_of_pos int32 [tiles * 64] (-1: padding), tile_expert int32 [tiles] (-1: none)."""
+    rows, experts = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1 or not logits.is_cuda:
+        raise KernelError("experts_route: float logits with contiguous rows")
+    tiles = tile_expert.shape[0]
+    if tiles < expert_tiles(rows, top, experts) or not 0 < top <= min(experts, 16):
+        raise KernelError(f"experts_route: {tiles} tiles for {rows} rows x {top} of {experts} experts")
+    _check(lib().cisr_experts_route(logits.data_ptr(), logits.stride(0), None if bias is None else _dev(bias, "bias", torch.float32, (experts,)),
+                                    _dev(chosen, "chosen", torch.int32, (rows, top)), _dev(weights, "weights", torch.float32, (rows, top)),
+                                    rows, experts, top, tiles, _dev(pair_of_pos, "pair_of_pos", torch.int32, (tiles * EXPERT_TILE,)),
+                                    _dev(tile_expert, "tile_expert", torch.int32, (tiles,)), _stream()), "experts_route")
+    return chosen, weights
+
+
+def experts_gemm(a, w, pair_of_pos, tile_expert, out, top=0, scatter=False, act=False):
+    """out[row of place] = act(a[row of place] . w[expert of the place's tile]^T) over the places that experts_route
+    laid out.  w [experts, N, K]; `top` > 0: a place's operand is row pair // top of `a` (the step's rows), else the
+    place's own row; `scatter`: the result goes to row `pair` of out, else to the place's own row.  `act`: relu(.)^2."""
+    experts, n, k = w.shape
+    tiles = tile_expert.shape[0]
+    places = tiles * EXPERT_TILE
+    if a.dtype != w.dtype or a.dim() != 2 or a.shape[1] != k or a.stride(1) != 1 or not w.is_contiguous():
+        raise KernelError("experts_gemm: operands of one dtype, [rows, K] against [experts, N, K]")
+    if out.dim() != 2 or out.shape[1] != n or not out.is_contiguous() or (a.dtype == torch.float32 and out.dtype != torch.float32):
+        raise KernelError("experts_gemm: out is [rows, N], float for float operands")
+    if pair_of_pos.numel() != places:
+        raise KernelError("experts_gemm: the places do not fit the tiles")
+    if (top <= 0 and a.shape[0] < places) or (not scatter and out.shape[0] < places):
+        raise KernelError("experts_gemm: operands by place need a row a place")
+    _check(lib().cisr_experts_gemm(_dev(a, "a") if a.is_contiguous() else a.data_ptr(), a.stride(0), _dev(w, "w"),
+                                   _dev(tile_expert, "tile_expert", torch.int32), _dev(pair_of_pos, "pair_of_pos", torch.int32),
+                                   int(top), int(bool(scatter)), _dev(out, "out"), out.stride(0), tiles, n, k, int(bool(act)),
+                                   _storage(a, "a"), _storage(out, "out"), _stream()), "experts_gemm")
+    return out
+
+
+def mingru_piece(rows, decode_only):
+    """Rows of a piece where the minimal gated unit's scan walks long segments in pieces side by side (0: a thread walks
+    a whole segment)."""
+    if decode_only or rows < 256:
+        return 0
+    return 64 if rows < 4096 else 128
+
+
+def mingru_scan(proj, bias_z, bias_x, state, seg_start, state_slots, out, width, piece=0, carry=None):
+    """Element by element over `width` channels: z = sigmoid(a + bias_z), c = cand(b + bias_x), S <- (1 - z) S + z c,
+    out = S silu(g), with [a | b | g] the first 3 width columns of proj (a float view with contiguous rows) and
+    cand(u) = u + 1/2 for u >= 0, sigmoid(u) below.  S: state float [slots, >= width] rows of a view, read from and
+    written back to each segment's slot.  `piece` > 0: segments are walked in pieces of that many rows (three
+    launches); carry float [2 * (rows // piece + segments) * width]."""
+    rows = proj.shape[0]
+    segments = state_slots.shape[0]
+    pp, ld = _rows_of(proj, "proj")
+    sp, sld = _rows_of(state, "state")
+    if proj.shape[1] < 3 * width or state.shape[1] < width or tuple(out.shape) != (rows, width):
+        raise KernelError("mingru_scan: shapes do not fit the width")
+    cp, pieces = None, 0
+    if piece > 0:
+        pieces = rows // piece + segments
+        if carry is None or carry.numel() < 2 * pieces * width:
+            raise KernelError("mingru_scan: pieces need a carry buffer")
+        cp = _dev(carry, "carry", torch.float32)
+    _check(_rec().cisr_mingru_scan(pp, ld, _dev(bias_z, "bias_z", torch.float32, (width,)), _dev(bias_x, "bias_x", torch.float32, (width,)),
+                                   sp, sld, _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
+                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), _dev(out, "out", None, (rows, width)),
+                                   rows, segments, width, int(piece), cp, pieces, _storage(out, "out"), _stream()), "mingru_scan")
     return out

@@ -93,6 +93,10 @@ class Model:
 
     def state_needs(self):
         needs = {}
+        own = self.embedding.state_need() if hasattr(self.embedding, "state_need") else None
+        if own is not None:       # (an embedding that looks at the token before keeps it in the request's state slot)
+            from ..parts.embedding import STATE_SITE
+            needs[STATE_SITE] = own
         for index, entry in enumerate(self.schedule):
             need = self.layers[entry.layer].state_need()
             if need is not None:

@@ -324,6 +324,118 @@ class LatentAttention(Mixer):
         return ctx.add_product(act, self.w_out, residual)
 
 
+class SigmoidAttention(Mixer):
+    """Grouped-query attention over the paged cache without a softmax: a visible key weighs sigmoid(q . k scale +
+    b_head), one number `<name>.pb`[head] added to the score, and the weights are not normed over the keys.  Queries
+    and keys are RMS-normed over the whole projection (all heads at once, a weight an element) before `position` turns
+    the first `position.rotary_dim` coordinates of every head in neighbouring pairs; keys and values may differ in
+    size (`dim`, `vdim`); a row sees itself and the `window` - 1 keys before it (None: all).
+
+    The pages hold heads of `pad` = max(dim, vdim) coordinates (rounded up to a multiple of 8), the rest zero, so the
+    framework's attention kernels run with their sigmoid law (`head_bias`) and nothing else changed.  `own_kv` False:
+    the layer has no key and value tensors and reads the cache another layer wrote.  `keep`: the window the layer's
+    own cache keeps, where layers that read it look further back than it does itself (None with a window: its own).
+    `ride(weight)`: further rows for the input product, whose float results are then `rider`.
+    `names`: the tensors' names under `name`."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm", "bias": "pb"}
+
+    def __init__(self, name, hidden, heads, kv_heads, dim, vdim, scale, eps, position, window=None, keep="own", own_kv=True,
+                 names=None, tuning=None):
+        if heads % kv_heads:
+            raise ValueError(f"{heads} query heads are not a multiple of {kv_heads} key/value heads")
+        self.pad = -(-max(dim, vdim) // 8) * 8
+        if self.pad > 256:
+            raise ValueError(f"head sizes {dim} / {vdim}: at most 256")
+        if not scale > 0:
+            raise ValueError("the score scale must be positive")
+        if getattr(position, "pairing", "split_half") != "interleaved" or position.rotary_dim > dim:
+            raise ValueError("the position part must turn neighbouring pairs of at most `dim` coordinates")
+        self.name, self.hidden, self.heads, self.kv_heads, self.dim, self.vdim = name, hidden, heads, kv_heads, dim, vdim
+        self.scale, self.eps, self.position, self.window, self.own_kv = float(scale), float(eps), position, window, bool(own_kv)
+        self.keep = window if keep == "own" else keep
+        if self.keep is not None and (window is None or window > self.keep):
+            raise ValueError("a layer's cache keeps at least the keys the layer itself looks back over")
+        self.names = {**self.NAMES, **(names or {})}
+        self.tuning = tuning or kernel.DEFAULT_TUNING
+        self.w_in = self.w_own = self.w_out = self.q_weight = self.k_weight = self.head_bias = self.rider = None
+        self.rider_rows = 0
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return kernel.kernel_units(self.pad, dtype, "sigmoid")
+
+    def step_arrays(self):
+        return [kernel.SingleRows(self.tuning.split_single_from), kernel.RowsLongestFirst()]
+
+    def cache_need(self):
+        return KVNeed(self.kv_heads, self.pad, self.keep) if self.own_kv else None
+
+    def cache_read(self):
+        return None if self.own_kv else KVNeed(self.kv_heads, self.pad, self.window)
+
+    def tensor_specs(self):
+        H, nh, nkv, D, V = self.hidden, self.heads, self.kv_heads, self.dim, self.vdim
+        specs = [TensorSpec(self._tensor("q"), (nh * D, H)), TensorSpec(self._tensor("q_norm"), (nh * D,), init="one_plus_normal")]
+        if self.own_kv:
+            specs += [TensorSpec(self._tensor("k"), (nkv * D, H)), TensorSpec(self._tensor("v"), (nkv * V, H)),
+                      TensorSpec(self._tensor("k_norm"), (nkv * D,), init="one_plus_normal")]
+        return specs + [TensorSpec(self._tensor("bias"), (nh,)), TensorSpec(self._tensor("o"), (H, nh * V))]
+
+    def _join(self, extra=None):
+        parts = list(self.w_own) + ([] if extra is None else [extra])
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:      # rows of the fused projection are a multiple of 8: zero rows at the end
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+
+    def bind(self, tensors, dtype):
+        self.w_own = [matrix_operand(tensors[self._tensor(p)], dtype) for p in (("q", "k", "v") if self.own_kv else ("q",))]
+        self.own_rows = sum(p.shape[0] for p in self.w_own)
+        self._join()
+        self.w_out = matrix_operand(tensors[self._tensor("o")], dtype)
+        self.q_weight = tensors[self._tensor("q_norm")].to(torch.float32).contiguous()
+        self.k_weight = tensors[self._tensor("k_norm")].to(torch.float32).contiguous() if self.own_kv else None
+        self.head_bias = tensors[self._tensor("bias")].to(torch.float32).contiguous()
+
+    def ride(self, weight):
+        self.rider_rows = weight.shape[0]
+        self._join(weight)
+
+    def prepare(self, device, dtype):
+        self.position.prepare(device, dtype)
+
+    def output(self, h, ctx, site):
+        """The mixer's result, float [T, hidden], without the residual sum."""
+        T = h.shape[0]
+        nh, nkv, D, V, pad = self.heads, self.kv_heads, self.dim, self.vdim, self.pad
+        gid, kcache, vcache = ctx.cache.pages_of_site(site)
+        view = ctx.kv[gid]
+        cos, sin = self.position.tables()
+        # queries, keys and values before their norm are float (the norms' statistics are): one product with float results
+        proj = ops.gemm(h, self.w_in, ctx.buffer("sattn.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        self.rider = proj[:, self.own_rows:self.own_rows + self.rider_rows] if self.rider_rows else None
+        q = ctx.buffer("sattn.q", (T, nh * pad), ctx.dtype)
+        if self.own_kv:
+            ops.whole_norm_rope_scatter(proj, self.q_weight, self.k_weight, ctx.positions, view.slots, cos, sin, q, kcache, vcache,
+                                        nh, nkv, D, V, pad, view.page_size, self.eps)
+        else:
+            ops.whole_norm_rope_scatter(proj, self.q_weight, None, ctx.positions, None, cos, sin, q, None, None,
+                                        nh, nkv, D, V, pad, view.page_size, self.eps)
+        out = ctx.buffer("sattn.out", (T, nh * pad), ctx.dtype)
+        kernel.paged_attention(ctx, q, nh * pad, kcache, vcache, view, out, nh, nkv, pad, self.window, self.scale,
+                               tuning=self.tuning, head_bias=self.head_bias)
+        act = out if pad == V else ops.head_gate(out, None, ctx.buffer("sattn.act", (T, nh * V), ctx.dtype), nh, V, pad)
+        return ops.gemm(act, self.w_out, ctx.buffer("sattn.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
+
+
 register_part("mixer", "attention", PagedAttention)
+register_part("mixer", "sigmoid_attention", SigmoidAttention)
 register_part("mixer", "latent_attention", LatentAttention)
 register_part("mixer", "normed_gated_attention", NormedGatedAttention)

@@ -91,6 +91,18 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class _Cast:
+    """Stands where a norm would in StepContext.leave_normed / take_normed for "the rows themselves in the activations'
+    type": whoever writes the residual stream (an embedding, a block that norms after the sum) may leave that copy for
+    the block whose sublayers read the stream itself."""
+
+    def __repr__(self):
+        return "CAST"
+
+
+CAST = _Cast()
+
+
 def matrix_operand(t, dtype):
     """A stored matrix as a GEMM operand of the compute dtype.  bf16 -> float
     widening is exact; a 32-bit matrix run in bf16 is rounded to nearest even by

@@ -1,9 +1,13 @@
 """Arrangement of parts in a layer.  PreNormBlock is the Llama arrangement
 (reference: runtime/model.py:106-119): x = x + mixer(norm1(x)); x = x + ffn(norm2(x)),
 the residual stream x kept in float.  SandwichBlock norms each sublayer's result as well
-and scales it: x = x + m norm1b(mixer(norm1(x))); x = x + m norm2b(ffn(norm2(x)))."""
+and scales it: x = x + m norm1b(mixer(norm1(x))); x = x + m norm2b(ffn(norm2(x))).  PostNormBlock norms after the
+sum, and its sublayers read the stream itself: x = norm1(a x + g1 mixer(x)); x = norm2(a x + g2 ffn(x)), with
+optional gates g = sigmoid(W x + b) element by element."""
+import torch
+
 from ..kernels import ops
-from .base import Part, register_part
+from .base import CAST, Part, TensorSpec, matrix_operand, register_part
 
 
 class PreNormBlock(Part):
@@ -180,5 +184,97 @@ class SandwichBlock(Part):
         return residual
 
 
+class PostNormBlock(Part):
+    """The norm after the sum: x <- norm1(alpha x + mixer(x)), then x <- norm2(alpha x + ffn(x)); the sublayers read x
+    itself (in the activations' type).  With `gated` each sublayer's result is first multiplied element by element by
+    sigmoid(W x + b), W = `<name>.<gate names[i]>` [H, H] and b = `<...>.b`.  The sum, the gate, the norm and the copy of
+    the new rows in the activations' type are one kernel (ops.gate_post_norm); a feed-forward that gives its result as
+    weighted rows (ops.WeightedRows: routed experts) has them summed on the way.  The gate's product rides in the
+    sublayer's own first product where the sublayer offers that (`ride(weight)`, then `rider` after `output`: a float view
+    [T, H]); otherwise it is a product of its own.  `ffn` None: a layer without a feed-forward (no second norm)."""
+
+    def __init__(self, name, hidden, mixer_norm, mixer, ffn_norm=None, ffn=None, alpha=1.0, gated=False, gate_names=("rg1", "rg2")):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward comes with the norm after it, or not at all")
+        for norm in (mixer_norm, ffn_norm):
+            if norm is not None and getattr(norm, "fusable_as", None) != "rms":
+                raise ValueError("the norm after a sum must be an RMS norm (weight, eps)")
+        if not hasattr(mixer, "output") or (ffn is not None and not hasattr(ffn, "output")):
+            raise ValueError("the sublayers of this arrangement must give their result without the residual sum (output)")
+        self.name, self.hidden, self.alpha, self.gated = name, hidden, float(alpha), bool(gated)
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        self.gate_names = tuple(gate_names)
+        self.gates = {}       # sublayer index -> (weight or None if it rides, bias float)
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def _gated(self):
+        return [(i, sub) for i, sub in enumerate((self.mixer, self.ffn)) if self.gated and sub is not None]
+
+    def tensor_specs(self):
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        for i, _ in self._gated():
+            gate = f"{self.name}.{self.gate_names[i]}"
+            specs += [TensorSpec(gate, (self.hidden, self.hidden)), TensorSpec(gate + ".b", (self.hidden,))]
+        return specs
+
+    def bind(self, tensors, dtype):
+        for p in self.parts():
+            p.bind(tensors, dtype)
+        for i, sub in self._gated():
+            gate = f"{self.name}.{self.gate_names[i]}"
+            weight = matrix_operand(tensors[gate], dtype)
+            bias = tensors[gate + ".b"].to(torch.float32).contiguous()
+            if hasattr(sub, "ride"):
+                sub.ride(weight)          # the sublayer's first product makes the gate's too
+                weight = None
+            self.gates[i] = (weight, bias)
+
+    def prepare(self, device, dtype):
+        for p in self.parts():
+            p.prepare(device, dtype)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def cache_read(self):
+        return self.mixer.cache_read() if hasattr(self.mixer, "cache_read") else None
+
+    def state_need(self):
+        return self.mixer.state_need()
+
+    def kernel_units(self, dtype):
+        return [u for p in self.parts() if hasattr(p, "kernel_units") for u in p.kernel_units(dtype)]
+
+    def step_arrays(self):
+        return [a for p in self.parts() if hasattr(p, "step_arrays") for a in p.step_arrays()]
+
+    def _sum_and_norm(self, x, h, result, which, sub, norm, ctx):
+        """x <- norm(alpha x + gate * result) in place; returns the new rows in the activations' type."""
+        if isinstance(result, ops.Partials):
+            raise TypeError("a sublayer of this arrangement gives finished rows (or weighted rows), no partial sums")
+        gate = bias = None
+        if which in self.gates:
+            weight, bias = self.gates[which]
+            gate = sub.rider if weight is None else ops.gemm(h, weight, ctx.buffer(f"post.gate{which}", x.shape, torch.float32), scratch=ctx.scratch)
+        cast = None if ctx.dtype == torch.float32 else ctx.buffer(f"post.cast{which}", x.shape, ctx.dtype)
+        ops.gate_post_norm(x, result, norm.weight, norm.eps, self.alpha, gate=gate, gate_bias=bias, cast=cast)
+        return x if cast is None else cast
+
+    def forward(self, residual, ctx, site):
+        ctx.next_norm = None          # (no product of this block is left to a later norm)
+        ctx.settle(residual)
+        h = ctx.take_normed(CAST, residual)
+        if h is None:
+            h = residual if ctx.dtype == torch.float32 else ops.f32_to_bf16(residual, ctx.buffer("post.cast", residual.shape, ctx.dtype))
+        h = self._sum_and_norm(residual, h, self.mixer.output(h, ctx, site), 0, self.mixer, self.mixer_norm, ctx)
+        if self.ffn is not None:
+            h = self._sum_and_norm(residual, h, self.ffn.output(h, ctx), 1, self.ffn, self.ffn_norm, ctx)
+        ctx.leave_normed(CAST, residual, h)
+        return residual
+
+
+register_part("block", "postnorm", PostNormBlock)
 register_part("block", "prenorm", PreNormBlock)
 register_part("block", "sandwich", SandwichBlock)

@@ -126,6 +126,81 @@ class DenseMLP(FeedForward):
         return ctx.add_product(self._activations(h, ctx), self.w_down, residual)
 
 
+class RoutedExperts(FeedForward):
+    """A mixture of `experts` small feed-forwards of which every row uses `top`: router logits W_r h + b in float, the
+    `top` largest chosen (the lowest index wins a tie), their weights the softmax over the chosen logits only; an
+    expert is W_down relu(W_up h)^2 without biases, and the result is the weighted sum of the chosen experts'.
+
+    The rows of a step are ordered by expert on the device (ops.experts_route) and each expert's matrix meets only its
+    own rows, in tiles (ops.experts_gemm); the down products are left as `top` rows a step row for the kernel that
+    adds the sublayer's result (ops.WeightedRows).  `ride(weight)`: further rows for the router's product, whose
+    float results are then `rider`.  `names`: (router, expert prefix, up, down), the tensors' names under `name`;
+    expert j's matrices are `<name>.<prefix>j.<up|down>`."""
+
+    def __init__(self, name, hidden, intermediate, experts, top, names=("router", "e", "up", "down")):
+        if not 0 < top <= min(experts, 16):
+            raise ValueError(f"{top} of {experts} experts: between 1 and min(experts, 16)")
+        self.name, self.hidden, self.intermediate, self.experts, self.top = name, hidden, intermediate, int(experts), int(top)
+        self.names = tuple(names)
+        self.rider, self.rider_rows = None, 0
+
+    def _expert(self, j, which):
+        return f"{self.name}.{self.names[1]}{j}.{self.names[2 + which]}"
+
+    def tensor_specs(self):
+        H, I, router = self.hidden, self.intermediate, f"{self.name}.{self.names[0]}"
+        specs = [TensorSpec(router, (self.experts, H)), TensorSpec(router + ".b", (self.experts,))]
+        for j in range(self.experts):
+            specs += [TensorSpec(self._expert(j, 0), (I, H)), TensorSpec(self._expert(j, 1), (H, I))]
+        return specs
+
+    def _join(self, extra=None):
+        parts = [self.w_router] + ([] if extra is None else [extra])
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+
+    def bind(self, tensors, dtype):
+        router = f"{self.name}.{self.names[0]}"
+        self.w_router = matrix_operand(tensors[router], dtype)
+        self.router_bias = tensors[router + ".b"].to(torch.float32).contiguous()
+        self._join()
+        self.w_up = torch.stack([matrix_operand(tensors[self._expert(j, 0)], dtype) for j in range(self.experts)]).contiguous()
+        self.w_down = torch.stack([matrix_operand(tensors[self._expert(j, 1)], dtype) for j in range(self.experts)]).contiguous()
+
+    def ride(self, weight):
+        self.rider_rows = weight.shape[0]
+        self._join(weight)
+
+    def output(self, h, ctx):
+        """The feed-forward's result as ops.WeightedRows (float [T * top, hidden] and the weights [T, top])."""
+        T, E, top = h.shape[0], self.experts, self.top
+        logits = ops.gemm(h, self.w_in, ctx.buffer("moe.logits", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        self.rider = logits[:, E:E + self.rider_rows] if self.rider_rows else None
+        tiles = ops.expert_tiles(T, top, E)
+        chosen, weights = ctx.buffer("moe.chosen", (T, top), torch.int32), ctx.buffer("moe.weights", (T, top), torch.float32)
+        places, tile_expert = ctx.buffer("moe.places", (tiles * ops.EXPERT_TILE,), torch.int32), ctx.buffer("moe.tiles", (tiles,), torch.int32)
+        ops.experts_route(logits[:, :E], self.router_bias, top, chosen, weights, places, tile_expert)
+        up = ops.experts_gemm(h, self.w_up, places, tile_expert, ctx.buffer("moe.up", (tiles * ops.EXPERT_TILE, self.intermediate), ctx.dtype),
+                              top=top, act=True)
+        down = ops.experts_gemm(up, self.w_down, places, tile_expert, ctx.buffer("moe.down", (T * top, self.hidden), torch.float32),
+                                scatter=True)
+        return ops.WeightedRows(down, weights, top)
+
+    def forward(self, h, residual, ctx, norm=None):
+        return _add_weighted(residual, self.output(h, ctx))
+
+
+def _add_weighted(residual, y):
+    """residual += sum_k weights[:, k] * rows[k]: for an arrangement that adds a feed-forward's result itself (torch's own
+    kernels: no arrangement of this package takes this way)."""
+    rows, dim = residual.shape
+    residual += (y.rows.view(rows, y.top, dim) * y.weights.unsqueeze(-1)).sum(dim=1)
+    return residual
+
+
+register_part("ffn", "routed_experts", RoutedExperts)
 register_part("ffn", "gated_mlp", GatedMLP)
 register_part("ffn", "dense_mlp", DenseMLP)
 register_part("ffn", "clamped_glu", ClampedGLU)

@@ -25,7 +25,11 @@ class RotaryEmbedding(Part):
         turns over `original` positions, rotary_dim * ln(original / (2 pi t)) / (2 ln theta), pairs up to
         lo = max(floor(turns(fast)), 0) keep their frequency, pairs from hi = min(ceil(turns(slow)), rotary_dim - 1) on
         turn `factor` times slower, those between go over linearly; cosines and sines are multiplied by
-        0.1 ln(factor) + 1."""
+        0.1 ln(factor) + 1.
+        `scaling` by wavelength (the rule of Llama 3.1): {"factor", "low", "high", "original"}.  A pair whose wavelength
+        2 pi / f is shorter than original / high keeps its frequency, one longer than original / low turns `factor`
+        times slower, one between goes over linearly in s = (original / wavelength - low) / (high - low):
+        (1 - s) f / factor + s f; cosines and sines keep their size."""
         if pairing not in ("split_half", "interleaved"):
             raise ValueError(f"pairing {pairing!r} is neither split_half nor interleaved")
         self.pairing = pairing
@@ -33,8 +37,16 @@ class RotaryEmbedding(Part):
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary size {self.rotary_dim} must be even and at most the head size {head_dim}")
-        self.scaling = None
-        if scaling is not None:
+        self.scaling = self.by_wavelength = None
+        if scaling is not None and ("low" in scaling or "high" in scaling):
+            missing = [k for k in ("factor", "low", "high", "original") if k not in scaling]
+            if missing:
+                raise ValueError(f"rotary scaling by wavelength lacks {missing}")
+            self.by_wavelength = {k: float(scaling[k]) for k in ("factor", "low", "high", "original")}
+            w = self.by_wavelength
+            if not (w["factor"] > 0 and w["original"] > 0 and 0 < w["low"] < w["high"]):
+                raise ValueError("rotary scaling by wavelength: factor and original positive, 0 < low < high")
+        elif scaling is not None:
             missing = [k for k in ("factor", "original", "fast", "slow") if k not in scaling]
             if missing:
                 raise ValueError(f"rotary scaling lacks {missing}")
@@ -48,6 +60,13 @@ class RotaryEmbedding(Part):
         half, dims = self.rotary_dim // 2, self.rotary_dim
         index = np.arange(half, dtype=np.float64)
         freq = np.float64(self.theta) ** (-index * 2.0 / dims)
+        if self.by_wavelength is not None:
+            w = self.by_wavelength
+            wavelength = 2.0 * math.pi / freq
+            share = np.clip((w["original"] / wavelength - w["low"]) / (w["high"] - w["low"]), 0.0, 1.0)
+            between = (1.0 - share) * freq / w["factor"] + share * freq
+            return np.where(wavelength < w["original"] / w["high"], freq,
+                            np.where(wavelength > w["original"] / w["low"], freq / w["factor"], between))
         s = self.scaling
         if s is None:
             return freq

@@ -18,6 +18,11 @@ the state in the cache manager's state slots, in float in every mode:
                          part of the state), q and k are made unit vectors per head, q scaled by dim^(-1/2); each
                          head's result RMS-normed, times silu of a gate projection, then the output projection.
 
+  MinGRU                 no heads and no matrix state: S_t = (1 - z_t) S_(t-1) + z_t c_t element by element over `width`
+                         channels, z_t = sigmoid(Wz h + bz), c_t = cand(Wx h + bx) with cand(u) = u + 1/2 for u >= 0 and
+                         sigmoid(u) below (the gates read the current token only); the result is Wo (S_t silu(Wg h)).
+                         A kernel of its own (ops.mingru_scan).
+
 The projections and the convolution's inputs are products with float results; decays, step sizes, gates of the
 recurrence and the norms are float arithmetic; the operands of the output projections are the compute dtype.
 """
@@ -252,6 +257,67 @@ class GatedDeltaRule(Mixer):
         return ctx.add_product(self._normed_result(h, ctx, site), self.w_out, residual)
 
 
+class MinGRU(Mixer):
+    """The minimal gated recurrent unit over `width` channels (see the module's text).  State: float [width] a request,
+    zero at the start.  `ride(weight)`: further rows for the input product, whose float results are then `rider`.
+    `names`: the tensors' names under `name` (biases are `<projection>.b`)."""
+
+    NAMES = {"z": "z", "x": "x", "gate": "g", "o": "o"}
+
+    def __init__(self, name, hidden, width, names=None):
+        self.name, self.hidden, self.width = name, hidden, int(width)
+        self.names = {**self.NAMES, **(names or {})}
+        self.rider, self.rider_rows = None, 0
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return [library.RECURRENCE]
+
+    def state_need(self):
+        return StateNeed((self.width,), "float32")
+
+    def tensor_specs(self):
+        H, W, t = self.hidden, self.width, self._tensor
+        return [TensorSpec(t("z"), (W, H)), TensorSpec(t("z") + ".b", (W,)), TensorSpec(t("x"), (W, H)), TensorSpec(t("x") + ".b", (W,)),
+                TensorSpec(t("gate"), (W, H)), TensorSpec(t("o"), (H, W))]
+
+    def _join(self, extra=None):
+        parts = list(self.w_own) + ([] if extra is None else [extra])
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+
+    def bind(self, tensors, dtype):
+        t = self._tensor
+        # one product with float results: [z | x | gate] (everything that enters the recurrence is float)
+        self.w_own = [matrix_operand(tensors[t(p)], dtype) for p in ("z", "x", "gate")]
+        self._join()
+        self.w_out = matrix_operand(tensors[t("o")], dtype)
+        self.bias_z, self.bias_x = _float(tensors[t("z") + ".b"]), _float(tensors[t("x") + ".b"])
+
+    def ride(self, weight):
+        self.rider_rows = weight.shape[0]
+        self._join(weight)
+
+    def output(self, h, ctx, site):
+        """The mixer's result, float [T, hidden], without the residual sum; moves the request's state on."""
+        T, W = h.shape[0], self.width
+        proj = ops.gemm(h, self.w_in, ctx.buffer("mingru.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        self.rider = proj[:, 3 * W:3 * W + self.rider_rows] if self.rider_rows else None
+        piece = ops.mingru_piece(T, ctx.decode_only)
+        carry = ctx.buffer("mingru.carry", (2 * (T // piece + ctx.n_segments) * W,), torch.float32) if piece else None
+        act = ops.mingru_scan(proj, self.bias_z, self.bias_x, ctx.cache.state_storage[site], ctx.seg_start, ctx.state_slots,
+                              ctx.buffer("mingru.act", (T, W), ctx.dtype), W, piece=piece, carry=carry)
+        return ops.gemm(act, self.w_out, ctx.buffer("mingru.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
+
+
 class SideBySide(Mixer):
     """Two mixers that read the same input; the result is half the sum of theirs, each RMS-normed over the model
     width with a weight of its own (`<name>.<first_out>` / `<name>.<second_out>`).  At most one of the two keeps pages
@@ -306,3 +372,4 @@ register_part("mixer", "gated_linear_attention", GatedLinearAttention)
 register_part("mixer", "state_space_duality", StateSpaceDuality)
 register_part("mixer", "side_by_side", SideBySide)
 register_part("mixer", "gated_delta_rule", GatedDeltaRule)
+register_part("mixer", "mingru", MinGRU)
