@@ -136,11 +136,15 @@ def sigmoid_attention(h, w, p, m, eps, keys_values):
 
 # -- feed-forward -------------------------------------------------------------------------------------------------
 
-def routed_experts(h, w, p, mlp):
+def routed_experts(h, w, p, mlp, margins=None):
     """Each token goes through the `top` experts with the largest router logits; their results are weighed by the
-    softmax over those logits only.  An expert is Wdown relu(Wup h)^2."""
+    softmax over those logits only.  An expert is Wdown relu(Wup h)^2.  `margins`: a list that receives, per token, how
+    far the last chosen logit lies above the first one left out (infinite where every expert is chosen)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     logits = linear(h, w[p + ".router"], w[p + ".router.b"])
+    if margins is not None:
+        ordered = -np.sort(-logits, axis=1)
+        margins.append(ordered[:, top - 1] - ordered[:, top] if E > top else np.full(h.shape[0], np.inf))
     out = np.zeros((h.shape[0], np.asarray(w[p + ".e0.down"]).shape[0]))
     for t in range(h.shape[0]):
         chosen = np.argsort(-logits[t], kind="stable")[:top]
@@ -154,8 +158,9 @@ def routed_experts(h, w, p, mlp):
 
 # -- the model ----------------------------------------------------------------------------------------------------
 
-def forward(cfg, w, tokens, layers_out=None):
-    """Logits [T, vocab] of a whole sequence.  `layers_out`: a list that receives the residual stream after every layer."""
+def forward(cfg, w, tokens, layers_out=None, margins=None):
+    """Logits [T, vocab] of a whole sequence.  `layers_out`: a list that receives the residual stream after every layer;
+    `margins`: a list that receives every router's margins (routed_experts)."""
     eps, alpha = cfg["norm"]["eps"], cfg["postln_alpha"]
     x = embed(tokens, w, cfg["embedding"])
     kept = {}
@@ -173,7 +178,7 @@ def forward(cfg, w, tokens, layers_out=None):
         y = y * sigmoid(linear(x, w[p + ".rg1"], w[p + ".rg1.b"]))
         x = rmsnorm(alpha * x + y, w[p + ".norm1"], eps)
         if layer.get("mlp") is not None:
-            y = routed_experts(x, w, p + ".mlp", layer["mlp"])
+            y = routed_experts(x, w, p + ".mlp", layer["mlp"], margins)
             y = y * sigmoid(linear(x, w[p + ".rg2"], w[p + ".rg2.b"]))
             x = rmsnorm(alpha * x + y, w[p + ".norm2"], eps)
         if layers_out is not None:
