@@ -283,7 +283,7 @@ def main():
     ap.add_argument("--check", type=int, default=1, choices=[0, 1], help="compare the timed way of running with the plain one first")
     ap.add_argument("--widths", default="1024,2048,4096", help="designs workload: model widths to time (comma separated)")
     ap.add_argument("--design-layers", type=int, default=4, help="designs workload: layers of each model")
-    ap.add_argument("--designs", default="llama,novosun,ditazen", help="designs workload: which designs to time (comma separated)")
+    ap.add_argument("--designs", default="llama,novosun,ditazen,noresun", help="designs workload: which designs to time (comma separated)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
@@ -388,7 +388,7 @@ def main():
 
 
 def design_configs(width, layers, context):
-    """A Llama, a Novosun and a Ditazen configuration of the same width, depth, feed-forward size and vocabulary.  The Novosun
+    """A Llama, a Novosun, a Ditazen and a Noresun configuration of the same width, depth and vocabulary.  The Novosun
     layers alternate: softmax attention (heads of 64 for keys, 128 for values, a quarter as many key/value heads) beside
     a state-space layer (inner size twice the width in heads of 64, 128 states, a convolution of 4 taps), then gated
     linear attention (key size half the width, value size the width, in heads of 128 x 256)."""
@@ -416,12 +416,24 @@ def design_configs(width, layers, context):
     rule = {"type": "delta", "mlp": dense, "mixer": {"heads": 2 * heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}}
     ditazen = {"architecture": "Ditazen", "vocab": vocab, "width": width, "logit_scale": 1.0, "norm": {"eps": 1e-5},
                "layers": [(first, rule, window, rule)[i % 4] for i in range(layers)], "max_positions": context}
-    return {"llama": llama, "novosun": novosun, "ditazen": ditazen}
+    # Noresun: attention with sigmoid weights over a window of 1,024 keys (heads of 128, a quarter as many key/value heads, half
+    # of a head turns), the minimal gated unit (as wide as the model), the same attention reading the first layer's keys, the
+    # unit again; every layer with 16 experts of 2 x width of which a row uses 2 (8 width^2 active feed-forward parameters a
+    # layer where Llama has 12, 64 in all)
+    moe = {"kind": "moe", "expert": {"ff": 2 * width}, "router": {"experts": 16, "top": 2}}
+    sig = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+           "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    unit = {"type": "mingru", "mixer": {"width": width}, "mlp": moe}
+    order = [{"type": "attention", "mixer": sig, "mlp": moe}, unit, {"type": "attention", "mixer": {**sig, "kv_from": 0}, "mlp": moe}, unit]
+    noresun = {"architecture": "Noresun", "vocab": vocab, "width": width, "postln_alpha": 2.0, "norm": {"eps": 1e-5},
+               "embedding": {"scale": float(width) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+               "layers": [order[i % 4] for i in range(layers)], "max_positions": context}
+    return {"llama": llama, "novosun": novosun, "ditazen": ditazen, "noresun": noresun}
 
 
 def designs(args):
-    """Prompt steps and decode steps of the Novosun and Ditazen designs beside the Llama design at equal width, depth, feed-forward
-    size and vocabulary (random weights drawn on the device): tokens a second of a whole prompt of --prompt tokens and
+    """Prompt steps and decode steps of the Novosun, Ditazen and Noresun designs beside the Llama design at equal width, depth
+    and vocabulary (random weights drawn on the device): tokens a second of a whole prompt of --prompt tokens and
     of decode steps of 1, 8 and 64 requests after such prompts, through the step function with captured programs and
     the greedy pick."""
     import statistics
@@ -475,7 +487,7 @@ def designs(args):
             result["prefill"] = {"tokens": prompt, "ms": round(pf * 1e3, 3), "tokens_per_s": round(prompt / pf, 1)}
             out.setdefault(str(width), {})[design] = result
             del runner, model
-    return {"metric": f"prompt and decode tokens/s of the Novosun and Ditazen designs beside Llama at equal width, {args.design_layers} layers",
+    return {"metric": f"prompt and decode tokens/s of the Novosun, Ditazen and Noresun designs beside Llama at equal width, {args.design_layers} layers",
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "steps": steps,
             "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "prompt_len": prompt,
             "execution": args.execution, "widths": out}
