@@ -85,12 +85,13 @@ arrange_kernel(const int* __restrict__ chosen, int pairs, int experts, int max_t
 extern "C" int cisr_experts_route(const float* logits, int ld, const float* bias, int* chosen, float* weights, int rows,
                                   int experts, int top, int max_tiles, int* pair_of_pos, int* tile_expert, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (experts <= 0 || top <= 0 || top > MAX_TOP || top > experts || experts > 4096 ||
-        (long long)max_tiles * EX_TILE < (long long)rows * top + (long long)experts * (EX_TILE - 1))
+    const bool arrange = pair_of_pos != nullptr;        // (null: the caller wants the choice only)
+    if (experts <= 0 || top <= 0 || top > MAX_TOP || top > experts || experts > 4096 || (arrange && (!tile_expert ||
+        (long long)max_tiles * EX_TILE < (long long)rows * top + (long long)experts * (EX_TILE - 1))))
         return (int)hipErrorInvalidValue;
     route_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(logits, ld, bias, chosen, weights, rows, experts, top);
     int err = CISR_LAUNCH_CHECK();
-    if (err) return err;
+    if (err || !arrange) return err;
     arrange_kernel<<<1, 1024, 3 * experts * sizeof(int), stream>>>(chosen, rows * top, experts, max_tiles, pair_of_pos, tile_expert);
     return CISR_LAUNCH_CHECK();
 }
@@ -179,11 +180,14 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-#define EX_BK 32
-#define EX_LD 40         // bf16 elements a tile row takes in LDS (80 bytes: 16-byte chunks, rows spread over the banks)
+#define EX_BK 64
+#define EX_BN 128
+#define EX_LD 72         // bf16 elements a tile row takes in LDS (144 bytes: 16-byte chunks, rows spread over the banks)
 
-// A block of four waves owns 64 places x 64 columns; wave w the places 16 w .. 16 w + 15 and all four column tiles.
-// Operands go global memory -> registers -> LDS (two buffers, one barrier a 32-deep step) -> matrix-core operands.
+// A block of four waves owns 64 places x 128 columns; wave (wm, wn) the places 32 wm .. 32 wm + 31 and the columns
+// 64 wn .. 64 wn + 63: 2 x 4 tiles of 16 x 16, sixteen matrix instructions a 64-deep step against six operand reads.
+// Operands go global memory -> registers -> LDS (two buffers, one barrier a step) -> matrix-core operands; the next
+// step's global loads are in flight while this one is multiplied.
 template <typename TC, int ACT>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const int* __restrict__ tile_expert,
@@ -192,53 +196,151 @@ expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
     const int e = tile_expert[tile];
     if (e < 0) return;
     __shared__ __attribute__((aligned(16))) bf16_t As[2][EX_TILE * EX_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][EX_TILE * EX_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][EX_BN * EX_LD];
     __shared__ int crow[EX_TILE];
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+    const int wm = wave / 2, wn = wave % 2;
     const int r = lane % 16, g = lane / 16;
-    const int lr = tid / 4, lc = (tid % 4) * 8;               // this thread's chunk of a tile: row, first k
-    const int n0 = blockIdx.y * EX_TILE;
-    const int pos = tile * EX_TILE + lr;
-    const TileRows mine = tile_rows(pos, pair_of_pos[pos], gather_div, scatter);
-    if (tid % 4 == 0) crow[lr] = mine.c;
-    const bf16_t* ap = mine.a >= 0 ? A + (size_t)mine.a * lda : nullptr;
-    const bf16_t* wp = n0 + lr < N ? W + ((size_t)e * N + n0 + lr) * K : nullptr;
-    const u32x4 zero = {0u, 0u, 0u, 0u};
-    auto fetch = [&](int k0, u32x4& va, u32x4& vw) {
-        const int k = k0 + lc;
-        va = (ap && k < K) ? *(const u32x4*)(ap + k) : zero;
-        vw = (wp && k < K) ? *(const u32x4*)(wp + k) : zero;
-    };
-    f32x4 acc[4];
+    const int lr = tid / 8, lc = (tid % 8) * 8;               // this thread's chunks of a tile: rows lr + 32 i, first k
+    const int n0 = blockIdx.y * EX_BN;
+    const bf16_t* ap[2];
+    const bf16_t* wp[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    u32x4 va, vw;
-    fetch(0, va, vw);
+    for (int i = 0; i < 2; ++i) {
+        const int pos = tile * EX_TILE + lr + 32 * i;
+        const TileRows mine = tile_rows(pos, pair_of_pos[pos], gather_div, scatter);
+        if (tid % 8 == 0) crow[lr + 32 * i] = mine.c;
+        ap[i] = mine.a >= 0 ? A + (size_t)mine.a * lda : nullptr;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int n = n0 + lr + 32 * i;
+        wp[i] = n < N ? W + ((size_t)e * N + n) * K : nullptr;
+    }
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    u32x4 va[2], vw[4];
+    auto fetch = [&](int k0) {
+        const int k = k0 + lc;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) va[i] = (ap[i] && k < K) ? *(const u32x4*)(ap[i] + k) : zero;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vw[i] = (wp[i] && k < K) ? *(const u32x4*)(wp[i] + k) : zero;
+    };
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    fetch(0);
     int buf = 0;
     for (int k0 = 0; k0 < K; k0 += EX_BK) {
-        *(u32x4*)(&As[buf][lr * EX_LD + lc]) = va;
-        *(u32x4*)(&Ws[buf][lr * EX_LD + lc]) = vw;
-        __syncthreads();       // whoever writes this buffer again, two steps on, has passed the next step's barrier
-        if (k0 + EX_BK < K) fetch(k0 + EX_BK, va, vw);
-        const bf16x8 fa = *(const bf16x8*)(&As[buf][(wave * 16 + r) * EX_LD + g * 8]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const bf16x8 fw = *(const bf16x8*)(&Ws[buf][(j * 16 + r) * EX_LD + g * 8]);
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fw, acc[j], 0, 0, 0);
+        for (int i = 0; i < 2; ++i) *(u32x4*)(&As[buf][(lr + 32 * i) * EX_LD + lc]) = va[i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(u32x4*)(&Ws[buf][(lr + 32 * i) * EX_LD + lc]) = vw[i];
+        __syncthreads();       // whoever writes this buffer again, two steps on, has passed the next step's barrier
+        if (k0 + EX_BK < K) fetch(k0 + EX_BK);
+#pragma unroll
+        for (int ks = 0; ks < EX_BK / 32; ++ks) {
+            bf16x8 fa[2], fw[4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = *(const bf16x8*)(&As[buf][(wm * 32 + i * 16 + r) * EX_LD + ks * 32 + g * 8]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fw[j] = *(const bf16x8*)(&Ws[buf][(wn * 64 + j * 16 + r) * EX_LD + ks * 32 + g * 8]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
         }
         buf ^= 1;
     }
     // a lane holds rows 4 g .. 4 g + 3 of column r in every 16 x 16 tile
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-        const int m = crow[wave * 16 + g * 4 + x];
-        if (m < 0) continue;
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int m = crow[wm * 32 + i * 16 + g * 4 + x];
+            if (m < 0) continue;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + wn * 64 + j * 16 + r;
+                if (n < N) store_f32(C + (size_t)m * ldc + n, expert_act<ACT>(acc[i][j][x]));
+            }
+        }
+}
+
+// ------------------------------------------------------------------ few rows: a pair streams its expert's matrix
+// Steps of few rows (decoding) are bound by the bytes of the chosen experts' matrices.  grid (N / 16, pairs): a block of
+// four waves makes 16 columns of one pair's row, a wave 4 of them: the operand row's share of a lane stays in registers
+// (K up to 64 x 8 x EX_ROW_CHUNKS), the four matrix rows are read 16 bytes a lane, all loads of a column quartet in
+// flight together.  C[pair] = act(A[pair / gather_div or pair] . W[chosen[pair]]^T).
+#define EX_ROW_CHUNKS 16
+template <typename TC, int ACT>
+__global__ void __launch_bounds__(256)
+expert_rows_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const int* __restrict__ chosen,
+                   int gather_div, TC* __restrict__ C, int ldc, int N, int K) {
+    const int pair = blockIdx.y;
+    const int e = chosen[pair];
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int n_first = (blockIdx.x * 4 + wave) * 4;
+    if (n_first >= N) return;
+    const bf16_t* ar = A + (size_t)(gather_div > 0 ? pair / gather_div : pair) * lda;
+    const int chunks = (K + 511) / 512;                      // 16-byte chunks a lane holds of a row
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    u32x4 av[EX_ROW_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < EX_ROW_CHUNKS; ++c) {
+        const int k = (c * 64 + lane) * 8;
+        av[c] = (c < chunks && k < K) ? *(const u32x4*)(ar + k) : zero;
+    }
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    const bf16_t* wr[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wr[j] = W + ((size_t)e * N + min(n_first + j, N - 1)) * K;
+#pragma unroll
+    for (int c = 0; c < EX_ROW_CHUNKS; ++c) {
+        if (c >= chunks) continue;                           // (uniform; the loop stays unrolled, the row in registers)
+        const int k = (c * 64 + lane) * 8;
+        u32x4 wv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wv[j] = k < K ? __builtin_nontemporal_load((const u32x4*)(wr[j] + k)) : zero;
+        const uint32_t aw[4] = {av[c].x, av[c].y, av[c].z, av[c].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int n = n0 + j * 16 + r;
-            if (n < N) store_f32(C + (size_t)m * ldc + n, expert_act<ACT>(acc[j][x]));
+            const uint32_t ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                sum[j] = fmaf(__uint_as_float(aw[x] << 16), __uint_as_float(ww[x] << 16), sum[j]);
+                sum[j] = fmaf(__uint_as_float(aw[x] & 0xffff0000u), __uint_as_float(ww[x] & 0xffff0000u), sum[j]);
+            }
         }
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum[j] = wave_sum(sum[j]);
+    if (lane < 4 && n_first + lane < N)
+        store_f32(C + (size_t)pair * ldc + n_first + lane, expert_act<ACT>(lane == 0 ? sum[0] : lane == 1 ? sum[1] : lane == 2 ? sum[2] : sum[3]));
+}
+
+// Whether cisr_experts_rows takes a product: bf16 operands with 16-byte rows of at most 64 x 8 x EX_ROW_CHUNKS elements.
+extern "C" int cisr_experts_rows_ok(int K, int lda, int pairs) {
+    return K % 8 == 0 && lda % 8 == 0 && K <= 512 * EX_ROW_CHUNKS && pairs > 0 && pairs <= 65535;
+}
+
+extern "C" int cisr_experts_rows(const void* A, int lda, const void* W, const int* chosen, int gather_div, void* C, int ldc,
+                                 int pairs, int N, int K, int act, int out_dtype, hipStream_t stream) {
+    if (pairs <= 0 || N <= 0) return 0;
+    if (!cisr_experts_rows_ok(K, lda, pairs) || ((uintptr_t)A) % 16 || ((uintptr_t)W) % 16) return (int)hipErrorInvalidValue;
+    const dim3 grid((N + 15) / 16, pairs);
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    if (out_dtype == DT_F32) {
+        if (act) expert_rows_kernel<float, 1><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (float*)C, ldc, N, K);
+        else expert_rows_kernel<float, 0><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (float*)C, ldc, N, K);
+    } else {
+        if (act) expert_rows_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (bf16_t*)C, ldc, N, K);
+        else expert_rows_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (bf16_t*)C, ldc, N, K);
+    }
+    return CISR_LAUNCH_CHECK();
 }
 
 // C[c row of place] = act(A[a row of place] . W[expert of the place's tile]^T); W is [experts, N, K].
@@ -251,6 +353,7 @@ extern "C" int cisr_experts_gemm(const void* A, int lda, const void* W, const in
     if (K <= 0 || max_tiles > 0x7fffff || (N + EX_TILE - 1) / EX_TILE > 65535 || (dtype == DT_F32 && out_dtype != DT_F32))
         return (int)hipErrorInvalidValue;
     const dim3 grid(max_tiles, (N + EX_TILE - 1) / EX_TILE);
+    const dim3 wide(max_tiles, (N + EX_BN - 1) / EX_BN);
 #define EX_ARGS tile_expert, pair_of_pos, gather_div, scatter
     if (dtype == DT_F32) {
         if (act) expert_gemm_fma_kernel<float, float, 1><<<grid, 256, 0, stream>>>((const float*)A, lda, (const float*)W, EX_ARGS, (float*)C, ldc, N, K);
@@ -262,11 +365,11 @@ extern "C" int cisr_experts_gemm(const void* A, int lda, const void* W, const in
     const bf16_t* w = (const bf16_t*)W;
     if (vec) {
         if (out_dtype == DT_F32) {
-            if (act) expert_gemm_mfma_kernel<float, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
-            else expert_gemm_mfma_kernel<float, 0><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+            if (act) expert_gemm_mfma_kernel<float, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+            else expert_gemm_mfma_kernel<float, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
         } else {
-            if (act) expert_gemm_mfma_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
-            else expert_gemm_mfma_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+            if (act) expert_gemm_mfma_kernel<bf16_t, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+            else expert_gemm_mfma_kernel<bf16_t, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
         }
     } else {
         if (out_dtype == DT_F32) {

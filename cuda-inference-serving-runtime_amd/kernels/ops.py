@@ -88,6 +88,8 @@ def _declare(h):
         "cisr_whole_norm_rope_scatter": [p, i, p, p, p, p, p, p, i, i, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_experts_route": [p, i, p, p, p, i, i, i, i, p, p, p],
         "cisr_experts_gemm": [p, i, p, p, p, i, i, p, i, i, i, i, i, i, i, p],
+        "cisr_experts_rows": [p, i, p, p, i, p, i, i, i, i, i, i, p],
+        "cisr_experts_rows_ok": [i, i, i],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -1452,21 +1454,50 @@ def expert_tiles(rows, top, experts):
     return -(-rows * top // EXPERT_TILE) + experts
 
 
-def experts_route(logits, bias, top, chosen, weights, pair_of_pos, tile_expert):
+def experts_route(logits, bias, top, chosen, weights, pair_of_pos=None, tile_expert=None):
     """logits: a float view [T, E] with unit column stride (+ bias float [E]) -> chosen int32 [T, top] (largest first,
-    the lowest index wins a tie), weights float [T, top] (softmax over the chosen logits), and the (row, choice) pairs
-    ordered by expert: pair_of_pos int32 [tiles * 64] (-1: padding), tile_expert int32 [tiles] (-1: none)."""
+    the lowest index wins a tie), weights float [T, top] (softmax over the chosen logits), and, unless pair_of_pos is
+    None, the (row, choice) pairs ordered by expert: pair_of_pos int32 [tiles * 64] (-1: padding), tile_expert int32
+    [tiles] (-1: none)."""
     rows, experts = logits.shape
     if logits.dtype != torch.float32 or logits.stride(1) != 1 or not logits.is_cuda:
         raise KernelError("experts_route: float logits with contiguous rows")
-    tiles = tile_expert.shape[0]
-    if tiles < expert_tiles(rows, top, experts) or not 0 < top <= min(experts, 16):
-        raise KernelError(f"experts_route: {tiles} tiles for {rows} rows x {top} of {experts} experts")
+    if not 0 < top <= min(experts, 16):
+        raise KernelError(f"experts_route: {top} of {experts} experts")
+    tiles, pp, tp = 0, None, None
+    if pair_of_pos is not None:
+        tiles = tile_expert.shape[0]
+        if tiles < expert_tiles(rows, top, experts):
+            raise KernelError(f"experts_route: {tiles} tiles for {rows} rows x {top} of {experts} experts")
+        pp, tp = _dev(pair_of_pos, "pair_of_pos", torch.int32, (tiles * EXPERT_TILE,)), _dev(tile_expert, "tile_expert", torch.int32, (tiles,))
     _check(lib().cisr_experts_route(logits.data_ptr(), logits.stride(0), None if bias is None else _dev(bias, "bias", torch.float32, (experts,)),
                                     _dev(chosen, "chosen", torch.int32, (rows, top)), _dev(weights, "weights", torch.float32, (rows, top)),
-                                    rows, experts, top, tiles, _dev(pair_of_pos, "pair_of_pos", torch.int32, (tiles * EXPERT_TILE,)),
-                                    _dev(tile_expert, "tile_expert", torch.int32, (tiles,)), _stream()), "experts_route")
+                                    rows, experts, top, tiles, pp, tp, _stream()), "experts_route")
     return chosen, weights
+
+
+EXPERT_ROWS_PAIRS = 32     # steps of at most this many (row, choice) pairs stream each pair's matrices (experts_rows)
+
+
+def experts_rows_ok(a, w, pairs):
+    """Whether experts_rows takes the product: bf16, few pairs, rows of 16-byte chunks that a wave holds in registers."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < pairs <= EXPERT_ROWS_PAIRS and a.stride(1) == 1
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and bool(lib().cisr_experts_rows_ok(int(w.shape[2]), int(a.stride(0)), int(pairs))))
+
+
+def experts_rows(a, w, chosen, out, top=0, act=False):
+    """out[pair] = act(a[pair // top, or pair with top 0] . w[chosen[pair]]^T) for every (row, choice) pair of a step of
+    few rows: a pair's block streams its expert's matrix (no layout by expert).  w [experts, N, K] bf16; chosen int32
+    [T, top] flattened to pairs; out [pairs, N]."""
+    experts, n, k = w.shape
+    pairs = chosen.numel()
+    if not experts_rows_ok(a, w, pairs) or a.shape[1] != k or tuple(out.shape) != (pairs, n) or not out.is_contiguous():
+        raise KernelError("experts_rows: shape not supported")
+    if a.shape[0] < (-(-pairs // top) if top > 0 else pairs):
+        raise KernelError("experts_rows: too few operand rows")
+    _check(lib().cisr_experts_rows(a.data_ptr(), a.stride(0), _dev(w, "w"), _dev(chosen, "chosen", torch.int32), int(top), _dev(out, "out"),
+                                   out.stride(0), pairs, n, k, int(bool(act)), _storage(out, "out"), _stream()), "experts_rows")
+    return out
 
 
 def experts_gemm(a, w, pair_of_pos, tile_expert, out, top=0, scatter=False, act=False):

@@ -178,14 +178,20 @@ class RoutedExperts(FeedForward):
         T, E, top = h.shape[0], self.experts, self.top
         logits = ops.gemm(h, self.w_in, ctx.buffer("moe.logits", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
         self.rider = logits[:, E:E + self.rider_rows] if self.rider_rows else None
-        tiles = ops.expert_tiles(T, top, E)
         chosen, weights = ctx.buffer("moe.chosen", (T, top), torch.int32), ctx.buffer("moe.weights", (T, top), torch.float32)
+        down = ctx.buffer("moe.down", (T * top, self.hidden), torch.float32)
+        if ops.experts_rows_ok(h, self.w_up, T * top) and ops.experts_rows_ok(h, self.w_down, T * top):
+            # few rows (decoding): every (row, choice) pair streams its expert's two matrices
+            ops.experts_route(logits[:, :E], self.router_bias, top, chosen, weights)
+            up = ops.experts_rows(h, self.w_up, chosen, ctx.buffer("moe.up", (T * top, self.intermediate), ctx.dtype), top=top, act=True)
+            ops.experts_rows(up, self.w_down, chosen, down)
+            return ops.WeightedRows(down, weights, top)
+        tiles = ops.expert_tiles(T, top, E)
         places, tile_expert = ctx.buffer("moe.places", (tiles * ops.EXPERT_TILE,), torch.int32), ctx.buffer("moe.tiles", (tiles,), torch.int32)
         ops.experts_route(logits[:, :E], self.router_bias, top, chosen, weights, places, tile_expert)
         up = ops.experts_gemm(h, self.w_up, places, tile_expert, ctx.buffer("moe.up", (tiles * ops.EXPERT_TILE, self.intermediate), ctx.dtype),
                               top=top, act=True)
-        down = ops.experts_gemm(up, self.w_down, places, tile_expert, ctx.buffer("moe.down", (T * top, self.hidden), torch.float32),
-                                scatter=True)
+        ops.experts_gemm(up, self.w_down, places, tile_expert, down, scatter=True)
         return ops.WeightedRows(down, weights, top)
 
     def forward(self, h, residual, ctx, norm=None):

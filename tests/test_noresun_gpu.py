@@ -116,7 +116,7 @@ def test_min_gru_scan_over_segments_with_states_carried_and_slots_used_again(wid
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows, experts, top, hidden, ff", [(1, 4, 1, 24, 16), (9, 5, 3, 20, 7), (150, 16, 2, 64, 40), (70, 3, 3, 100, 12)])
+@pytest.mark.parametrize("rows, experts, top, hidden, ff", [(1, 4, 1, 24, 16), (9, 5, 3, 20, 7), (150, 16, 2, 64, 40), (70, 3, 3, 100, 12), (8, 6, 2, 1040, 520)])
 def test_routed_experts_route_and_products(dtype, rows, experts, top, hidden, ff):
     """Choice and weights against a plain top-k (with a tie that the lower index wins); the layout by expert holds every
     pair once, in its expert's tiles; both products against plain arithmetic of the same operands."""
@@ -158,6 +158,16 @@ def test_routed_experts_route_and_products(dtype, rows, experts, top, hidden, ff
         ex = want.reshape(-1)[pair]
         close(upn[pos], np.maximum(uf[ex] @ hf[pair // top], 0.0) ** 2, tol)
         close(down[pair].cpu().numpy(), df[ex] @ upn[pos], tol)
+    if ops.experts_rows_ok(h, w_up, rows * top) and ops.experts_rows_ok(up, w_down, rows * top):
+        # steps of few rows: every pair streams its expert's matrices; the same numbers without the layout by expert
+        up2 = ops.experts_rows(h, w_up, chosen, torch.empty(rows * top, ff, dtype=td, device="cuda"), top=top, act=True)
+        down2 = ops.experts_rows(up2, w_down, chosen, torch.full((rows * top, hidden), float("nan"), device="cuda"))
+        for pair in range(rows * top):
+            ex = want.reshape(-1)[pair]
+            close(up2[pair].double().cpu().numpy(), np.maximum(uf[ex] @ hf[pair // top], 0.0) ** 2, tol)
+            close(down2[pair].cpu().numpy(), df[ex] @ up2[pair].double().cpu().numpy(), tol)
+    else:
+        assert dtype == "float32" or rows * top > ops.EXPERT_ROWS_PAIRS or hidden % 8 or ff % 8
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
