@@ -191,8 +191,17 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 template <typename TC, int ACT>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const int* __restrict__ tile_expert,
-                        const int* __restrict__ pair_of_pos, int gather_div, int scatter, TC* __restrict__ C, int ldc, int N, int K) {
-    const int tile = blockIdx.x;
+                        const int* __restrict__ pair_of_pos, int gather_div, int scatter, TC* __restrict__ C, int ldc, int N, int K,
+                        int tiles) {
+    // The hardware deals consecutive blocks round-robin to the 8 XCDs, each with an L2 of its own.  Renumber so that an
+    // XCD gets a contiguous run of (tile, column block) pairs, tiles fastest: the tiles of one expert follow each other,
+    // so the blocks that read the same 128 rows of that expert's matrix run on one XCD at about the same time.
+    // The grid is one row of blocks, rounded up to a multiple of 8.
+    const int blocks = tiles * ((N + EX_BN - 1) / EX_BN);
+    const int per_xcd = (blocks + 7) / 8;
+    const int slot = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
+    if (slot >= blocks) return;
+    const int tile = slot % tiles, column_block = slot / tiles;
     const int e = tile_expert[tile];
     if (e < 0) return;
     __shared__ __attribute__((aligned(16))) bf16_t As[2][EX_TILE * EX_LD];
@@ -202,7 +211,7 @@ expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
     const int wm = wave / 2, wn = wave % 2;
     const int r = lane % 16, g = lane / 16;
     const int lr = tid / 8, lc = (tid % 8) * 8;               // this thread's chunks of a tile: rows lr + 32 i, first k
-    const int n0 = blockIdx.y * EX_BN;
+    const int n0 = column_block * EX_BN;
     const bf16_t* ap[2];
     const bf16_t* wp[4];
 #pragma unroll
@@ -353,7 +362,9 @@ extern "C" int cisr_experts_gemm(const void* A, int lda, const void* W, const in
     if (K <= 0 || max_tiles > 0x7fffff || (N + EX_TILE - 1) / EX_TILE > 65535 || (dtype == DT_F32 && out_dtype != DT_F32))
         return (int)hipErrorInvalidValue;
     const dim3 grid(max_tiles, (N + EX_TILE - 1) / EX_TILE);
-    const dim3 wide(max_tiles, (N + EX_BN - 1) / EX_BN);
+    const long long wide_blocks = (long long)max_tiles * ((N + EX_BN - 1) / EX_BN);
+    if (wide_blocks > 0x7ffffff0LL) return (int)hipErrorInvalidValue;
+    const dim3 wide((unsigned)((wide_blocks + 7) / 8 * 8));
 #define EX_ARGS tile_expert, pair_of_pos, gather_div, scatter
     if (dtype == DT_F32) {
         if (act) expert_gemm_fma_kernel<float, float, 1><<<grid, 256, 0, stream>>>((const float*)A, lda, (const float*)W, EX_ARGS, (float*)C, ldc, N, K);
@@ -365,11 +376,11 @@ extern "C" int cisr_experts_gemm(const void* A, int lda, const void* W, const in
     const bf16_t* w = (const bf16_t*)W;
     if (vec) {
         if (out_dtype == DT_F32) {
-            if (act) expert_gemm_mfma_kernel<float, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
-            else expert_gemm_mfma_kernel<float, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);
+            if (act) expert_gemm_mfma_kernel<float, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K, max_tiles);
+            else expert_gemm_mfma_kernel<float, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K, max_tiles);
         } else {
-            if (act) expert_gemm_mfma_kernel<bf16_t, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
-            else expert_gemm_mfma_kernel<bf16_t, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K);
+            if (act) expert_gemm_mfma_kernel<bf16_t, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K, max_tiles);
+            else expert_gemm_mfma_kernel<bf16_t, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K, max_tiles);
         }
     } else {
         if (out_dtype == DT_F32) {

@@ -412,7 +412,8 @@ def test_prompt_then_tokens_one_by_one_and_portions_down_to_two_tokens(folders, 
     runner.cache.check()
 
 
-def test_a_long_portion_walked_in_pieces(folders):
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_portion_walked_in_pieces(folders, dtype):
     """A portion long enough for the recurrent unit's scan to walk it in pieces side by side, after a shorter one that
     leaves a state, beside a second request's portion in the same step."""
     from runtime.engine import StepEntry
@@ -421,12 +422,12 @@ def test_a_long_portion_walked_in_pieces(folders):
     V = CONFIGS[name]["vocab"]
     long, other = random_tokens(31, 700, V), random_tokens(32, 300, V)
     assert ops.mingru_piece(600 + 300, False) > 0
-    runner = make_runner(folders[name], "float32", pages=70)
+    runner = make_runner(folders[name], dtype, pages=70)
     runner.create("l"); runner.create("o")
     got = [runner.step([StepEntry("l", long[:100], list(range(100)))]).cpu().numpy()]
     out = runner.step([StepEntry("l", long[100:], list(range(600))), StepEntry("o", other, list(range(300)))]).cpu().numpy()
-    assert_close(np.concatenate([got[0], out[:600]]), plain_logits(folders[name], long), "float32", "pieces")
-    assert_close(out[600:], plain_logits(folders[name], other), "float32", "the second request")
+    assert_close(np.concatenate([got[0], out[:600]]), plain_logits(folders[name], long), dtype, "pieces", decided_rows(folders[name], long))
+    assert_close(out[600:], plain_logits(folders[name], other), dtype, "the second request", decided_rows(folders[name], other))
 
 
 @pytest.mark.parametrize("name, dtype, execution", [("b", "float32", "graph"), ("a", "bfloat16", "graph"), ("s", "float32", "eager")])
