@@ -426,7 +426,7 @@ def design_configs(width, layers, context):
     unit = {"type": "mingru", "mixer": {"width": width}, "mlp": moe}
     order = [{"type": "attention", "mixer": sig, "mlp": moe}, unit, {"type": "attention", "mixer": {**sig, "kv_from": 0}, "mlp": moe}, unit]
     noresun = {"architecture": "Noresun", "vocab": vocab, "width": width, "postln_alpha": 2.0, "norm": {"eps": 1e-5},
-               "embedding": {"scale": float(width) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+               "embedding": {"scale": float(width) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 131, "mul_cur": 17}},
                "layers": [order[i % 4] for i in range(layers)], "max_positions": context}
     return {"llama": llama, "novosun": novosun, "ditazen": ditazen, "noresun": noresun}
 

@@ -173,3 +173,28 @@ def decided_rows(folder, tokens):
     than the float64 implementation does, which is no fault; such a position is compared in float32 only.  (A close
     call also reaches later positions through the recurrent state and the cached keys, but thinly: they stay in.)"""
     return _plain(folder, tokens)[1] >= CLOSE_CALL
+
+
+def smallest_margins(folder, tokens):
+    """For every position the smallest margin by which a router of the plain model decides there."""
+    return _plain(folder, tokens)[1]
+
+
+FLIP = 0.01           # a margin below which the rounding of a bfloat16 run that has come some layers far may choose otherwise
+
+
+def decisive_tokens(folder, seed, n, vocab, margin=FLIP, tries=200):
+    """`n` token ids drawn from `seed` at none of whose positions a router of the plain model decides by less than
+    `margin`: the first position that does gets another token until none is left (a position's routers see only the
+    tokens up to it, so what is settled stays settled).  A choice that bfloat16 rounding turns round changes the keys
+    and states that later positions read, and no comparison should rest on one."""
+    rng = np.random.default_rng(seed)
+    tokens = [int(t) for t in rng.integers(0, vocab, n)]
+    for _ in range(tries):
+        margins = _plain(folder, tokens)[1]
+        close = np.nonzero(margins < margin)[0]
+        if not len(close):
+            return tokens
+        _PLAIN.pop((str(folder), tuple(tokens)), None)
+        tokens[int(close[0])] = int(rng.integers(0, vocab))
+    raise AssertionError(f"no sequence of {n} tokens without a close call after {tries} tries")
