@@ -182,13 +182,17 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 #define EX_BK 64
 #define EX_BN 128
+#define EX_PAIRED_FROM 48   // tiles a step can take from which a block takes two tiles of one expert at a time
 #define EX_LD 72         // bf16 elements a tile row takes in LDS (144 bytes: 16-byte chunks, rows spread over the banks)
 
-// A block of four waves owns 64 places x 128 columns; wave (wm, wn) the places 32 wm .. 32 wm + 31 and the columns
-// 64 wn .. 64 wn + 63: 2 x 4 tiles of 16 x 16, sixteen matrix instructions a 64-deep step against six operand reads.
-// Operands go global memory -> registers -> LDS (two buffers, one barrier a step) -> matrix-core operands; the next
-// step's global loads are in flight while this one is multiplied.
-template <typename TC, int ACT>
+// A block of four waves owns 64 MT places x 128 columns; wave (wm, wn) the places 32 MT wm .. 32 MT wm + 32 MT - 1 and
+// the columns 64 wn .. 64 wn + 63: 2 MT x 4 tiles of 16 x 16, 16 MT matrix instructions a 64-deep step against 2 MT + 4
+// operand reads.  Operands go global memory -> registers -> LDS (two buffers, one barrier a step) -> matrix-core
+// operands; the next step's global loads (MT 1: the next two steps') are in flight while this one is multiplied.
+// MT 2 (steps of many rows): the block of a tile that is the first, third, ... of its expert's run also takes the tile
+// after it if that is the same expert's (else its second half is padding), and the block of the other tile leaves at
+// once: every byte of the expert's matrix then meets twice the rows.
+template <typename TC, int ACT, int MT>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const int* __restrict__ tile_expert,
                         const int* __restrict__ pair_of_pos, int gather_div, int scatter, TC* __restrict__ C, int ldc, int N, int K,
@@ -204,21 +208,29 @@ expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
     const int tile = slot % tiles, column_block = slot / tiles;
     const int e = tile_expert[tile];
     if (e < 0) return;
-    __shared__ __attribute__((aligned(16))) bf16_t As[2][EX_TILE * EX_LD];
+    int places = EX_TILE;              // places of this block that are not padding by construction
+    if (MT == 2) {
+        int before = 0;                // tiles of this expert's run before this one
+        while (tile - before - 1 >= 0 && tile_expert[tile - before - 1] == e) ++before;
+        if (before & 1) return;
+        if (tile + 1 < tiles && tile_expert[tile + 1] == e) places = 2 * EX_TILE;
+    }
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][MT * EX_TILE * EX_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[2][EX_BN * EX_LD];
-    __shared__ int crow[EX_TILE];
+    __shared__ int crow[MT * EX_TILE];
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
     const int wm = wave / 2, wn = wave % 2;
     const int r = lane % 16, g = lane / 16;
     const int lr = tid / 8, lc = (tid % 8) * 8;               // this thread's chunks of a tile: rows lr + 32 i, first k
     const int n0 = column_block * EX_BN;
-    const bf16_t* ap[2];
+    const bf16_t* ap[2 * MT];
     const bf16_t* wp[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int pos = tile * EX_TILE + lr + 32 * i;
-        const TileRows mine = tile_rows(pos, pair_of_pos[pos], gather_div, scatter);
-        if (tid % 8 == 0) crow[lr + 32 * i] = mine.c;
+    for (int i = 0; i < 2 * MT; ++i) {
+        const int row = lr + 32 * i;
+        const int pos = tile * EX_TILE + row;
+        const TileRows mine = tile_rows(pos, row < places ? pair_of_pos[pos] : -1, gather_div, scatter);
+        if (tid % 8 == 0) crow[row] = mine.c;
         ap[i] = mine.a >= 0 ? A + (size_t)mine.a * lda : nullptr;
     }
 #pragma unroll
@@ -227,48 +239,60 @@ expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
         wp[i] = n < N ? W + ((size_t)e * N + n) * K : nullptr;
     }
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    u32x4 va[2], vw[4];
-    auto fetch = [&](int k0) {
+    // MT 1: two steps' operands are on their way at any time (two sets of registers taking turns: one step's arithmetic
+    // is shorter than a trip to the L2); MT 2 has registers for one set, and more arithmetic a step
+    u32x4 va0[2 * MT], vw0[4], va1[2 * MT], vw1[4];
+    auto fetch = [&](int k0, u32x4 (&va)[2 * MT], u32x4 (&vw)[4]) {
         const int k = k0 + lc;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) va[i] = (ap[i] && k < K) ? *(const u32x4*)(ap[i] + k) : zero;
+        for (int i = 0; i < 2 * MT; ++i) va[i] = (ap[i] && k < K) ? *(const u32x4*)(ap[i] + k) : zero;
 #pragma unroll
         for (int i = 0; i < 4; ++i) vw[i] = (wp[i] && k < K) ? *(const u32x4*)(wp[i] + k) : zero;
     };
-    f32x4 acc[2][4];
+    f32x4 acc[2 * MT][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2 * MT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    fetch(0);
     int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += EX_BK) {
+    // one 64-deep step: the set's operands into LDS, the set asked for again `ahead` steps on, the step multiplied
+    auto step = [&](int k0, u32x4 (&va)[2 * MT], u32x4 (&vw)[4], int ahead) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *(u32x4*)(&As[buf][(lr + 32 * i) * EX_LD + lc]) = va[i];
+        for (int i = 0; i < 2 * MT; ++i) *(u32x4*)(&As[buf][(lr + 32 * i) * EX_LD + lc]) = va[i];
 #pragma unroll
         for (int i = 0; i < 4; ++i) *(u32x4*)(&Ws[buf][(lr + 32 * i) * EX_LD + lc]) = vw[i];
         __syncthreads();       // whoever writes this buffer again, two steps on, has passed the next step's barrier
-        if (k0 + EX_BK < K) fetch(k0 + EX_BK);
+        if (k0 + ahead * EX_BK < K) fetch(k0 + ahead * EX_BK, va, vw);
 #pragma unroll
         for (int ks = 0; ks < EX_BK / 32; ++ks) {
-            bf16x8 fa[2], fw[4];
+            bf16x8 fa[2 * MT], fw[4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) fa[i] = *(const bf16x8*)(&As[buf][(wm * 32 + i * 16 + r) * EX_LD + ks * 32 + g * 8]);
+            for (int i = 0; i < 2 * MT; ++i) fa[i] = *(const bf16x8*)(&As[buf][(wm * 32 * MT + i * 16 + r) * EX_LD + ks * 32 + g * 8]);
 #pragma unroll
             for (int j = 0; j < 4; ++j) fw[j] = *(const bf16x8*)(&Ws[buf][(wn * 64 + j * 16 + r) * EX_LD + ks * 32 + g * 8]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2 * MT; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
         }
         buf ^= 1;
+    };
+    fetch(0, va0, vw0);
+    if (MT == 1) {
+        if (EX_BK < K) fetch(EX_BK, va1, vw1);
+        for (int k0 = 0; k0 < K; k0 += 2 * EX_BK) {
+            step(k0, va0, vw0, 2);
+            if (k0 + EX_BK < K) step(k0 + EX_BK, va1, vw1, 2);
+        }
+    } else {
+        for (int k0 = 0; k0 < K; k0 += EX_BK) step(k0, va0, vw0, 1);
     }
     // a lane holds rows 4 g .. 4 g + 3 of column r in every 16 x 16 tile
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2 * MT; ++i)
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-            const int m = crow[wm * 32 + i * 16 + g * 4 + x];
+            const int m = crow[wm * 32 * MT + i * 16 + g * 4 + x];
             if (m < 0) continue;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -375,13 +399,18 @@ extern "C" int cisr_experts_gemm(const void* A, int lda, const void* W, const in
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
     if (vec) {
+        // steps of many rows (an expert meets more than one tile as a rule): a block takes two tiles of one expert
+#define EX_MFMA(TC, ACT) \
+        do { if (max_tiles >= EX_PAIRED_FROM) expert_gemm_mfma_kernel<TC, ACT, 2><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (TC*)C, ldc, N, K, max_tiles); \
+             else expert_gemm_mfma_kernel<TC, ACT, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (TC*)C, ldc, N, K, max_tiles); } while (0)
         if (out_dtype == DT_F32) {
-            if (act) expert_gemm_mfma_kernel<float, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K, max_tiles);
-            else expert_gemm_mfma_kernel<float, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K, max_tiles);
+            if (act) EX_MFMA(float, 1);
+            else EX_MFMA(float, 0);
         } else {
-            if (act) expert_gemm_mfma_kernel<bf16_t, 1><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K, max_tiles);
-            else expert_gemm_mfma_kernel<bf16_t, 0><<<wide, 256, 0, stream>>>(a, lda, w, EX_ARGS, (bf16_t*)C, ldc, N, K, max_tiles);
+            if (act) EX_MFMA(bf16_t, 1);
+            else EX_MFMA(bf16_t, 0);
         }
+#undef EX_MFMA
     } else {
         if (out_dtype == DT_F32) {
             if (act) expert_gemm_fma_kernel<bf16_t, float, 1><<<grid, 256, 0, stream>>>(a, lda, w, EX_ARGS, (float*)C, ldc, N, K);

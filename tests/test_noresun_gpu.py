@@ -116,10 +116,13 @@ def test_min_gru_scan_over_segments_with_states_carried_and_slots_used_again(wid
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows, experts, top, hidden, ff", [(1, 4, 1, 24, 16), (9, 5, 3, 20, 7), (150, 16, 2, 64, 40), (70, 3, 3, 100, 12), (8, 6, 2, 1040, 520)])
+@pytest.mark.parametrize("rows, experts, top, hidden, ff", [(1, 4, 1, 24, 16), (9, 5, 3, 20, 7), (150, 16, 2, 64, 40), (70, 3, 3, 100, 12), (8, 6, 2, 1040, 520),
+                                                             (1100, 6, 3, 72, 136), (3000, 20, 1, 64, 48)])
 def test_routed_experts_route_and_products(dtype, rows, experts, top, hidden, ff):
     """Choice and weights against a plain top-k (with a tie that the lower index wins); the layout by expert holds every
-    pair once, in its expert's tiles; both products against plain arithmetic of the same operands."""
+    pair once, in its expert's tiles; both products against plain arithmetic of the same operands.  The last two
+    cases have rows enough for the form in which a block takes two tiles of one expert (runs of odd and even length, a
+    product deeper than a whole number of steps)."""
     from runtime.kernels import ops
     rng = np.random.default_rng(rows + experts)
     td = TORCH[dtype]
@@ -151,7 +154,7 @@ def test_routed_experts_route_and_products(dtype, rows, experts, top, hidden, ff
     down = torch.full((rows * top, hidden), float("nan"), device="cuda")
     ops.experts_gemm(up, w_down, places, tile_expert, down, scatter=True)
     hf, uf, df = h.double().cpu().numpy(), w_up.double().cpu().numpy(), w_down.double().cpu().numpy()
-    upn = up.double().cpu().numpy()
+    upn, down = up.double().cpu().numpy(), down.cpu()
     tol = 1e-5 if dtype == "float32" else 1e-2
     for pos in np.nonzero(pl >= 0)[0]:
         pair = pl[pos]
