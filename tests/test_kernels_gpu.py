@@ -1052,8 +1052,8 @@ def test_product_left_unfinished_is_added_by_the_norm_that_follows(ops, M, monke
 
 
 def test_library_products_of_many_rows_also_in_captured_graphs(ops, monkeypatch):
-    """Large bf16 products of many rows may go to the vendor's library, with the residual sum and the activation
-    as kernels after it.  Checked against float products, eagerly and in a captured graph that is replayed with
+    """Large bf16 products of many rows may go to the vendor's library (with bf16 or with float results), with the
+    residual sum and the activation as kernels after it.  Checked against float products, eagerly and in a captured graph that is replayed with
     new inputs, eager work and synchronisations between the replays (a library call may record nodes that go
     wrong on later replays: every replay is checked)."""
     monkeypatch.setattr(ops, "LIBRARY_MIN_ROWS", 256)
@@ -1068,15 +1068,18 @@ def test_library_products_of_many_rows_also_in_captured_graphs(ops, monkeypatch)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     res = torch.empty(M, N, device=DEV)
     act = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+    out_f = torch.empty(M, N, device=DEV)
 
     def step():
         ops.gemm(a, w, out)
+        ops.gemm(a, w, out_f)           # float results: the library's float accumulators as they are, nothing rounded
         ops.gemm(a, w, res, residual=res)
         ops.gemm_swiglu(a, w_gu, act)
 
     def check(tag):
         ref = a.float() @ w.float().T
         torch.testing.assert_close(out.float(), ref, rtol=2e-2, atol=2e-2, msg=tag)
+        assert ((out_f.double() - a.double() @ w.double().T).abs().max() / ref.abs().max()).item() < 1e-5, tag
         torch.testing.assert_close(res - r0, ref, rtol=2e-2, atol=2e-2, msg=tag)   # the product is rounded to bf16 before the sum
         gq = (a.float() @ w_gu.float().T).bfloat16().float()
         torch.testing.assert_close(act.float(), torch.nn.functional.silu(gq[:, :I]) * gq[:, I:], rtol=2e-2, atol=2e-3, msg=tag)
@@ -1090,7 +1093,7 @@ def test_library_products_of_many_rows_also_in_captured_graphs(ops, monkeypatch)
         step()
     for i in range(5):
         a.copy_(torch.randn(M, K, device=DEV) * 0.5); res.copy_(r0)
-        out.fill_(7); act.fill_(7)
+        out.fill_(7); act.fill_(7); out_f.fill_(7)
         junk = (torch.randn(300, 300, device=DEV) @ torch.randn(300, 300, device=DEV)).sum().item()   # eager work between replays
         graph.replay()
         torch.cuda.synchronize()
