@@ -422,7 +422,7 @@ def design_configs(width, layers, context):
     # layer where Llama has 12, 64 in all)
     moe = {"kind": "moe", "expert": {"ff": 2 * width}, "router": {"experts": 16, "top": 2}}
     sig = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
-           "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+           "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
     unit = {"type": "mingru", "mixer": {"width": width}, "mlp": moe}
     order = [{"type": "attention", "mixer": sig, "mlp": moe}, unit, {"type": "attention", "mixer": {**sig, "kv_from": 0}, "mlp": moe}, unit]
     noresun = {"architecture": "Noresun", "vocab": vocab, "width": width, "postln_alpha": 2.0, "norm": {"eps": 1e-5},
