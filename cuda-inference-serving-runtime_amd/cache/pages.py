@@ -57,6 +57,18 @@ class KVNeed:
 
 
 @dataclass(frozen=True)
+class ChunkNeed(KVNeed):
+    """Keys and values of a mixer whose rows see only their own block of `chunk` positions (blocks counted from
+    position 0, up to the row itself).  `window` = `chunk` bounds what a request holds; what can be given back is more
+    than a window's rule says: once a request's next token starts a block, every page before that block is dead."""
+    chunk: int = 0
+
+    def first_visible(self, length):
+        """The first position that the token at `length`, or any later one, can see."""
+        return length // self.chunk * self.chunk if self.chunk > 0 else 0
+
+
+@dataclass(frozen=True)
 class StateNeed:
     """A fixed-size state per request."""
     shape: tuple
@@ -114,6 +126,9 @@ class CacheGroup:
     # -- planning -------------------------------------------------------
     def _dead_pages(self, request, length):
         """Logical pages that no later query can see (window groups only)."""
+        rule = getattr(self.need, "first_visible", None)
+        if rule is not None:               # (a need with a rule of its own: blocks of positions)
+            return rule(length) // self.page_size
         if self.need.window is None:
             return 0
         first_visible = max(0, length - self.need.window + 1)  # the next token sits at `length`

@@ -4,4 +4,5 @@ from .llama import LlamaConfig
 from .novosun import NovosunConfig
 from .ditazen import DitazenConfig
 from .noresun import NoresunConfig
+from .zovozen import ZovozenConfig
 from .presets import preset, preset_names

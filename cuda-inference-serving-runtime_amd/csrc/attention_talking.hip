@@ -1,0 +1,214 @@
+// Attention whose scores are mixed over the heads before the softmax, over the paged cache: one block a token row,
+// all query heads of the row together.
+//
+//   raw_g(j)  = q_g . k_kv(g)(j)                                   for every query head g and visible key j
+//   s_h(j)    = sum_g mix[h, g] temp[g] scale raw_g(j)             (the heads' scores talk to each other)
+//   w_h(j)    = exp(s_h(j)) / (exp(sink_h) + sum_j' exp(s_h(j')))  (a sink: a term of the denominator without a key)
+//   out_h     = sum_j w_h(j) v_kv(h)(j)    [times sigmoid(gate) element by element]
+//
+// A row at position p sees the keys lo..p of its request: lo = (p / chunk) chunk with `chunk` > 0 (blocks of positions
+// counted from 0 that see only themselves), p - window + 1 with `window` > 0, else 0.  Its own key is in the cache before
+// this kernel runs.  Exact float arithmetic on float or bf16 storage (scores, the mix, the softmax and the sums are
+// float); the pages hold heads of `pad` coordinates whose rest is zero (keys [pages, kv_heads, page_size, pad], values
+// transposed in a page), queries come as [rows, heads * pad].
+//
+// Keys are walked 64 at a time, tiles at absolute multiples of 64: (1) a thread a (key head, key) makes the raw scores
+// of the head's group, 16 bytes of the key row a load; (2) a thread a (head, key) mixes; (3) a wave a head moves the
+// running maximum and denominator; (4) a thread an output coordinate (E of them in registers) adds the tile's values,
+// eight keys of a transposed value page a load where pages hold a multiple of eight keys.
+#include "common.h"
+
+#define TK_KEYS 64
+
+struct TalkArgs {
+    const void* q; int q_row_stride;
+    const void* kcache; const void* vcache;
+    const int* tables; const int* seg_of_row; const int* positions;
+    const float* mix; const float* temp; const float* sink;
+    const float* gate; int ldg;
+    void* out;
+    int heads, kv_heads, vdim, pad, page_size, width, window, chunk;
+    float scale;
+};
+
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 a = *(const uint4*)p;
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+}
+
+template <typename T, int E>
+__global__ void __launch_bounds__(256)
+attn_talking_kernel(TalkArgs p) {
+    extern __shared__ float lds[];
+    const int H = p.heads, G = p.kv_heads, pad = p.pad, P = p.page_size, group = H / G;
+    float* qs = lds;                          // [H, pad]
+    float* mixw = qs + H * pad;               // [H, H]: mix[h, g] temp[g] scale
+    float* raw = mixw + H * H;                // [H, 64]
+    float* pw = raw + H * TK_KEYS;            // [H, 64]
+    float* run_m = pw + H * TK_KEYS;          // [H]
+    float* run_l = run_m + H;                 // [H]
+    float* alpha = run_l + H;                 // [H]
+    int* pg = (int*)(alpha + H);              // [64]: the page of a key of the tile (-1: not visible)
+    int* po = pg + TK_KEYS;                   // [64]: its place in the page
+
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int seg = p.seg_of_row[row];
+    const int n_out = H * p.vdim;
+    T* out = (T*)p.out + (size_t)row * n_out;
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[e] = 0.f;
+    int begin = 0, end = 0;
+    if (seg >= 0) {
+        const int pos = p.positions[row];
+        end = pos + 1;
+        begin = p.chunk > 0 ? (pos / p.chunk) * p.chunk : (p.window > 0 && end > p.window) ? end - p.window : 0;
+    }
+    if (begin >= end) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) { const int i = tid + 256 * e; if (i < n_out) store_f32(out + i, 0.f); }
+        return;
+    }
+    const T* qr = (const T*)p.q + (size_t)row * p.q_row_stride;
+    for (int i = tid; i < H * pad; i += 256) qs[i] = load_f32(qr + i);
+    for (int i = tid; i < H * H; i += 256) mixw[i] = p.mix[i] * (p.temp ? p.temp[i % H] : 1.0f) * p.scale;
+    for (int h = tid; h < H; h += 256) {
+        run_m[h] = p.sink ? p.sink[h] : -INFINITY;        // the sink: a key of score sink_h and no value
+        run_l[h] = p.sink ? 1.0f : 0.f;
+    }
+    const int* table = p.tables + (size_t)seg * p.width;
+    const T* kc = (const T*)p.kcache;
+    const T* vc = (const T*)p.vcache;
+    const bool by8 = P % 8 == 0;
+    for (int base = begin / TK_KEYS * TK_KEYS; base < end; base += TK_KEYS) {
+        __syncthreads();                      // (the tile before is done with pg, po, pw, alpha; the first: qs, mixw are there)
+        if (tid < TK_KEYS) {
+            const int t = base + tid;
+            const bool seen = t >= begin && t < end;
+            pg[tid] = seen ? table[t / P] : -1;
+            po[tid] = t % P;
+        }
+        __syncthreads();
+        // (1) raw scores of a key head's group of query heads, four heads at a time
+        for (int item = tid; item < G * TK_KEYS; item += 256) {
+            const int c = item / TK_KEYS, j = item % TK_KEYS;
+            if (pg[j] < 0) continue;
+            const T* kr = kc + (((size_t)pg[j] * G + c) * P + po[j]) * pad;
+            for (int g0 = 0; g0 < group; g0 += 4) {
+                float dot[4] = {0.f, 0.f, 0.f, 0.f};
+                const float* q0 = qs + (size_t)(c * group + g0) * pad;
+                for (int d = 0; d < pad; d += 8) {
+                    float kv[8];
+                    load8(kr + d, kv);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (g0 + u < group) {
+                            const float* qh = q0 + u * pad + d;
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) dot[u] += qh[i] * kv[i];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) if (g0 + u < group) raw[(c * group + g0 + u) * TK_KEYS + j] = dot[u];
+            }
+        }
+        __syncthreads();
+        // (2) the mix over the heads
+        for (int item = tid; item < H * TK_KEYS; item += 256) {
+            const int h = item / TK_KEYS, j = item % TK_KEYS;
+            float s = -INFINITY;
+            if (pg[j] >= 0) {
+                s = 0.f;
+                for (int g = 0; g < H; ++g) s += mixw[h * H + g] * raw[g * TK_KEYS + j];
+            }
+            pw[item] = s;
+        }
+        __syncthreads();
+        // (3) running maximum and denominator, a wave a head
+        for (int h = wave; h < H; h += 4) {
+            const float s = pw[h * TK_KEYS + lane];
+            const float m_old = run_m[h];
+            const float m_new = fmaxf(m_old, wave_max(s));          // finite: the tile has a visible key
+            const float w = expf(s - m_new);                        // exp(-inf) = 0
+            const float a = expf(m_old - m_new);
+            const float l = run_l[h] * a + wave_sum(w);
+            pw[h * TK_KEYS + lane] = w;
+            if (lane == 0) { run_m[h] = m_new; run_l[h] = l; alpha[h] = a; }
+        }
+        __syncthreads();
+        // (4) the values
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int i = tid + 256 * e;
+            if (i >= n_out) continue;
+            const int h = i / p.vdim, d = i % p.vdim, c = h / group;
+            float a = acc[e] * alpha[h];
+            const float* wr = pw + h * TK_KEYS;
+            if (by8) {
+                for (int j = 0; j < TK_KEYS; j += 8) {
+                    int page = -1;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) page = max(page, pg[j + u]);      // (eight keys from a multiple of eight: one page)
+                    if (page < 0) continue;
+                    float vv[8];
+                    load8(vc + (((size_t)page * G + c) * pad + d) * P + po[j], vv);
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) a += wr[j + u] * vv[u];
+                }
+            } else {
+                for (int j = 0; j < TK_KEYS; ++j)
+                    if (pg[j] >= 0) a += wr[j] * load_f32(vc + (((size_t)pg[j] * G + c) * pad + d) * P + po[j]);
+            }
+            acc[e] = a;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int i = tid + 256 * e;
+        if (i >= n_out) continue;
+        const float l = run_l[i / p.vdim];
+        float v = l > 0.f ? acc[e] / l : 0.f;
+        if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)row * p.ldg + i]));
+        store_f32(out + i, v);
+    }
+}
+
+static size_t talking_lds(int heads, int pad) {
+    return ((size_t)heads * pad + (size_t)heads * heads + 2 * (size_t)heads * TK_KEYS + 3 * (size_t)heads) * sizeof(float) + 2 * TK_KEYS * sizeof(int);
+}
+
+template <typename T>
+static int launch_talking(const TalkArgs& a, int rows, hipStream_t stream) {
+    const size_t lds = talking_lds(a.heads, a.pad);
+    const int per = (a.heads * a.vdim + 255) / 256;
+#define TALK(E) attn_talking_kernel<T, E><<<rows, 256, lds, stream>>>(a)
+    if (per <= 2) TALK(2);
+    else if (per <= 4) TALK(4);
+    else if (per <= 8) TALK(8);
+    else if (per <= 16) TALK(16);
+    else if (per <= 32) TALK(32);
+    else return (int)hipErrorInvalidValue;
+#undef TALK
+    return CISR_LAUNCH_CHECK();
+}
+
+extern "C" int cisr_attn_talking(const void* q, int q_row_stride, const void* kcache, const void* vcache, const int* tables,
+                                 const int* seg_of_row, const int* positions, const float* mix, const float* temp, const float* sink,
+                                 const float* gate, int ldg, void* out, int rows, int heads, int kv_heads, int vdim, int pad,
+                                 int page_size, int width, int window, int chunk, float scale, int dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || pad <= 0 || pad % 8 || vdim <= 0 || vdim > pad || page_size <= 0 ||
+        !mix || talking_lds(heads, pad) > 64 * 1024 || q_row_stride < heads * pad || (gate && ldg < heads * vdim))
+        return (int)hipErrorInvalidValue;
+    const TalkArgs a = {q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, mix, temp, sink, gate, ldg, out,
+                        heads, kv_heads, vdim, pad, page_size, width, window, chunk, scale};
+    return dtype == DT_F32 ? launch_talking<float>(a, rows, stream) : launch_talking<bf16_t>(a, rows, stream);
+}

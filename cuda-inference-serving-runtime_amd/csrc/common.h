@@ -79,10 +79,12 @@ __device__ __forceinline__ float gated_activation(float g, float u, const GateLa
 
 // An ungated activation, the epilogue of a product that feeds a feed-forward's second matrix:
 //   1: z Phi(z), the gelu with the error function     2: its tanh form 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
-enum { ACT_NONE = 0, ACT_GELU = 1, ACT_GELU_TANH = 2 };
+//   3: relu(z)^2
+enum { ACT_NONE = 0, ACT_GELU = 1, ACT_GELU_TANH = 2, ACT_RELU2 = 3 };
 
 __device__ __forceinline__ float unary_activation(float z, int act) {
     if (act == ACT_GELU) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    if (act == ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
     return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
 }
 

@@ -9,14 +9,17 @@
 #include "common.h"
 
 // ------------------------------------------------- norm of a sublayer's output, scaled, into the residual stream
-// One block a row.  TWO: the row is half the sum of two rows, each normed over the width with a weight of its own.
-// With next_w the norm that reads the residual stream next is made on the way: next_out = rmsnorm(x) * next_w.
+// One block a row.  TWO: the row is half the sum of two rows, each normed over the width with a weight of its own; or,
+// without those weights (wa null), the plain sum ca a + cb b of the two rows.
+// With next_out the norm that reads the residual stream next is made on the way: next_out = rmsnorm(x) * next_w, or with
+// next_w null the new row itself in the activations' type (for sublayers that read the stream as it is).
 // KEEP: the row waits in LDS between the passes (rows of up to 16,384 floats); else it is read again.
 template <bool TWO, bool KEEP, typename T>
 __global__ void __launch_bounds__(256)
 post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
                      const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
-                     int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out) {
+                     int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out,
+                     float ca, float cb) {
     __shared__ float red[4];
     extern __shared__ float kept[];
     const size_t row = blockIdx.x;
@@ -31,11 +34,11 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
     }
     float ra = 1.f, rb = 0.f;
     if (TWO) {
-        ra = 0.5f / sqrtf(block_sum<256>(sa, red) / (float)dim + eps);
-        rb = 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps);
+        ra = wa ? 0.5f / sqrtf(block_sum<256>(sa, red) / (float)dim + eps) : ca;
+        rb = wa ? 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps) : cb;
         sa = 0.f;
         for (int d = threadIdx.x; d < dim; d += 256) {
-            const float y = ar[d] * ra * wa[d] + br[d] * rb * wb[d];
+            const float y = ar[d] * ra * (wa ? wa[d] : 1.0f) + br[d] * rb * (wa ? wb[d] : 1.0f);
             if (KEEP) kept[d] = y;
             sa += y * y;
         }
@@ -45,16 +48,16 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
     float* xr = x + row * dim;
     float sn = 0.f;
     for (int d = threadIdx.x; d < dim; d += 256) {         // (a thread reads back only what it wrote itself)
-        const float y = KEEP ? kept[d] : TWO ? ar[d] * ra * wa[d] + br[d] * rb * wb[d] : ar[d];
+        const float y = KEEP ? kept[d] : TWO ? ar[d] * ra * (wa ? wa[d] : 1.0f) + br[d] * rb * (wa ? wb[d] : 1.0f) : ar[d];
         const float xn = xr[d] + y * scale * (w ? w[d] : 1.0f);
         xr[d] = xn;
         if (KEEP) kept[d] = xn;
         sn += xn * xn;
     }
-    if (next_w == nullptr) return;
-    const float rs = 1.0f / sqrtf(block_sum<256>(sn, red) / (float)dim + next_eps);
+    if (next_out == nullptr) return;
+    const float rs = next_w ? 1.0f / sqrtf(block_sum<256>(sn, red) / (float)dim + next_eps) : 1.0f;
     T* out = next_out + row * dim;
-    for (int d = threadIdx.x; d < dim; d += 256) store_f32(out + d, (KEEP ? kept[d] : xr[d]) * rs * next_w[d]);
+    for (int d = threadIdx.x; d < dim; d += 256) store_f32(out + d, (KEEP ? kept[d] : xr[d]) * rs * (next_w ? next_w[d] : 1.0f));
 }
 
 // The same for rows of up to 4,096 floats: a thread holds E elements of every operand in registers, so that all of a
@@ -65,7 +68,7 @@ __global__ void __launch_bounds__(256)
 post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
                            const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
                            int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out,
-                           int slices_a, int slices_b) {
+                           int slices_a, int slices_b, float ca, float cb) {
     __shared__ float red[4];
     const size_t row = blockIdx.x;
     float va[E], vb[E], vx[E], vw[E], vwa[E], vwb[E], vn[E];
@@ -77,8 +80,8 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
         va[e] = in ? a[row * dim + dd] : 0.f;
         vx[e] = in ? x[row * dim + dd] : 0.f;
         vw[e] = w ? w[dd] : 1.f;
-        vn[e] = next_w ? next_w[dd] : 0.f;
-        if (TWO) { vb[e] = in ? b[row * dim + dd] : 0.f; vwa[e] = wa[dd]; vwb[e] = wb[dd]; }
+        vn[e] = next_w ? next_w[dd] : 1.f;
+        if (TWO) { vb[e] = in ? b[row * dim + dd] : 0.f; vwa[e] = wa ? wa[dd] : 1.f; vwb[e] = wa ? wb[dd] : 1.f; }
     }
     // the further slices of a cut product, four slices' loads on their way at a time, added in slice order
     auto add_slices = [&](float (&v)[E], const float* parts, int slices) {
@@ -103,8 +106,8 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
 #pragma unroll
     for (int e = 0; e < E; ++e) { sa += va[e] * va[e]; if (TWO) sb += vb[e] * vb[e]; }
     if (TWO) {
-        const float ra = 0.5f / sqrtf(block_sum<256>(sa, red) / (float)dim + eps);
-        const float rb = 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps);
+        const float ra = wa ? 0.5f / sqrtf(block_sum<256>(sa, red) / (float)dim + eps) : ca;
+        const float rb = wa ? 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps) : cb;
         sa = 0.f;
 #pragma unroll
         for (int e = 0; e < E; ++e) { va[e] = va[e] * ra * vwa[e] + vb[e] * rb * vwb[e]; sa += va[e] * va[e]; }
@@ -117,8 +120,8 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
         vx[e] += va[e] * scale * vw[e];
         if (d < dim) { x[row * dim + d] = vx[e]; sn += vx[e] * vx[e]; }
     }
-    if (next_w == nullptr) return;
-    const float rs = 1.0f / sqrtf(block_sum<256>(sn, red) / (float)dim + next_eps);
+    if (next_out == nullptr) return;
+    const float rs = next_w ? 1.0f / sqrtf(block_sum<256>(sn, red) / (float)dim + next_eps) : 1.0f;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int d = threadIdx.x + 256 * e;
@@ -129,29 +132,29 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
 template <bool TWO, typename T>
 static void launch_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb, const float* w,
                                  int rows, int dim, float eps, float mult, const float* next_w, float next_eps, T* next_out,
-                                 int slices_a, int slices_b, hipStream_t stream) {
-#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, slices_a, slices_b)
+                                 int slices_a, int slices_b, float ca, float cb, hipStream_t stream) {
+#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, slices_a, slices_b, ca, cb)
     if (dim <= 1024) SHORT(4);
     else if (dim <= 2048) SHORT(8);
     else if (dim <= 4096) SHORT(16);
 #undef SHORT
-    else if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
-    else post_norm_add_kernel<TWO, false, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
+    else if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, ca, cb);
+    else post_norm_add_kernel<TWO, false, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, ca, cb);
 }
 
 extern "C" int cisr_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb,
                                   const float* w, int rows, int dim, float eps, float mult, const float* next_w, float next_eps,
-                                  void* next_out, int next_dtype, int slices_a, int slices_b, hipStream_t stream) {
+                                  void* next_out, int next_dtype, int slices_a, int slices_b, float ca, float cb, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (dim <= 0 || (b != nullptr && (wa == nullptr || wb == nullptr)) || (next_w != nullptr && next_out == nullptr) ||
+    if (dim <= 0 || (b != nullptr && ((wa == nullptr) != (wb == nullptr))) || (next_w != nullptr && next_out == nullptr) ||
         slices_a < 0 || slices_b < 0 || ((slices_a > 0 || slices_b > 0) && dim > 4096))    // (partial sums: the kernel of short rows)
         return (int)hipErrorInvalidValue;
     if (next_dtype == DT_F32) {
-        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, stream);
-        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, stream);
+        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, ca, cb, stream);
+        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, ca, cb, stream);
     } else {
-        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, stream);
-        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, stream);
+        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, ca, cb, stream);
+        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, ca, cb, stream);
     }
     return CISR_LAUNCH_CHECK();
 }

@@ -261,16 +261,33 @@ extern "C" int cisr_heads_product(const void* a, int lda, int a_head, const void
 }
 
 // ------------------------------------------------------------------------------------------------ activation
-// kind 0: the form with the error function; kind 1: the tanh form (unary_activation of common.h)
+// kind 0: the gelu with the error function; kind 1: its tanh form; kind 2: relu(z)^2 (unary_activation of common.h)
 template <typename T>
 __global__ void __launch_bounds__(256) gelu_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n, int kind) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) store_f32(out + i, unary_activation(load_f32(x + i), kind == 0 ? ACT_GELU : ACT_GELU_TANH));
+    if (i < n) store_f32(out + i, unary_activation(load_f32(x + i), kind + 1));
+}
+
+// out = act(x + bias[column]) for a product whose bias keeps the activation out of its epilogue; the sum is float
+template <typename T>
+__global__ void __launch_bounds__(256) bias_act_kernel(const T* __restrict__ x, const float* __restrict__ bias, T* __restrict__ out,
+                                                       size_t n, int cols, int kind) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) store_f32(out + i, unary_activation(load_f32(x + i) + bias[i % cols], kind + 1));
+}
+
+extern "C" int cisr_bias_act(const void* x, const float* bias, void* out, long long n, int cols, int kind, int dtype, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (kind < 0 || kind > 2 || cols <= 0 || !bias) return (int)hipErrorInvalidValue;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == DT_F32) bias_act_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, bias, (float*)out, (size_t)n, cols, kind);
+    else bias_act_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, bias, (bf16_t*)out, (size_t)n, cols, kind);
+    return CISR_LAUNCH_CHECK();
 }
 
 extern "C" int cisr_gelu(const void* x, void* out, long long n, int kind, int dtype, hipStream_t stream) {
     if (n <= 0) return 0;
-    if (kind != 0 && kind != 1) return (int)hipErrorInvalidValue;
+    if (kind < 0 || kind > 2) return (int)hipErrorInvalidValue;
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == DT_F32) gelu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, (size_t)n, kind);
     else gelu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, (size_t)n, kind);

@@ -121,46 +121,64 @@ extern "C" int cisr_gate_post_norm(float* x, const float* y, int top, const floa
 }
 
 // ------------------------------------------------------------------ queries and keys normed over the whole projection
-// One block a row of a projection with float results [q: heads x dim | k: kv_heads x dim | v: kv_heads x vdim | ...]:
-// q and k are RMS-normed over all their heads at once (a weight an element), the first 2 `half` coordinates of every
-// head turn in neighbouring pairs (2i, 2i + 1) by the position's angles (cos / sin float [max_pos, half]); q goes to
-// q_out [T, heads * pad], k and v into the pages at `slots` as heads of `pad` coordinates, the rest zero (keys
-// [pages, kv_heads, page_size, pad], values transposed in a page).  has_kv 0: the row has queries only.
+// One block a row of a projection with float results [q: heads x dim | k: kv_heads x dim | v: kv_heads x vdim | ...]
+// (`bias`: float over these columns, added first, or null): q and k are RMS-normed over all their heads at once (a
+// weight an element), the first 2 `half` coordinates of every head turn by the position's angles (cos / sin float
+// [max_pos, half]) in neighbouring pairs (2i, 2i + 1), or with `split_half` in pairs (i, i + half); q goes to q_out
+// [T, heads * pad], k and v into the pages at `slots` as heads of `pad` coordinates, the rest zero (keys [pages,
+// kv_heads, page_size, pad], values transposed in a page).  `value_norm`: each head's value is divided by its root mean
+// square over vdim first (no weight).  has_kv 0: the row has queries only.
+#define WN_MAX_KV_HEADS 256
 template <typename T>
 __global__ void __launch_bounds__(256)
-whole_norm_rope_scatter_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ qw, const float* __restrict__ kw,
-                               const int* __restrict__ positions, const int* __restrict__ slots, const float* __restrict__ cosines,
-                               const float* __restrict__ sines, int half, int max_pos, T* __restrict__ q_out, T* __restrict__ kcache,
-                               T* __restrict__ vcache, int heads, int kv_heads, int dim, int vdim, int pad, int page_size, float eps,
-                               int has_kv) {
+whole_norm_rope_scatter_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ bias, const float* __restrict__ qw,
+                               const float* __restrict__ kw, const int* __restrict__ positions, const int* __restrict__ slots,
+                               const float* __restrict__ cosines, const float* __restrict__ sines, int half, int max_pos,
+                               T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache, int heads, int kv_heads, int dim,
+                               int vdim, int pad, int page_size, float eps, int has_kv, int split_half, int value_norm) {
     __shared__ float red[4];
+    __shared__ float rv[WN_MAX_KV_HEADS];
     const size_t row = blockIdx.x;
     const float* pr = proj + row * ld;
     const int nq = heads * dim, nk = kv_heads * dim;
+    auto val = [&](int i) { return bias ? pr[i] + bias[i] : pr[i]; };
     float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < nq; i += 256) { const float v = pr[i]; sq += v * v; }
+    for (int i = threadIdx.x; i < nq; i += 256) { const float v = val(i); sq += v * v; }
     const float rq = 1.0f / sqrtf(block_sum<256>(sq, red) / (float)nq + eps);
     float rk = 0.f;
     if (has_kv) {
-        for (int i = threadIdx.x; i < nk; i += 256) { const float v = pr[nq + i]; sk += v * v; }
+        for (int i = threadIdx.x; i < nk; i += 256) { const float v = val(nq + i); sk += v * v; }
         rk = 1.0f / sqrtf(block_sum<256>(sk, red) / (float)nk + eps);
+        if (value_norm) {
+            const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+            for (int h = wave; h < kv_heads; h += 4) {
+                float sv = 0.f;
+                for (int c = lane; c < vdim; c += WAVE) { const float v = val(nq + nk + h * vdim + c); sv += v * v; }
+                sv = wave_sum(sv);
+                if (lane == 0) rv[h] = 1.0f / sqrtf(sv / (float)vdim + eps);
+            }
+            __syncthreads();
+        }
     }
     int p = positions[row];
     p = p < 0 ? 0 : p >= max_pos ? max_pos - 1 : p;
     const float* cr = cosines + (size_t)p * half;
     const float* sr = sines + (size_t)p * half;
-    // coordinate c of a head of the normed vector src (weights wt), turned if it lies among the turning ones
-    auto turned = [&](const float* src, const float* wt, int base, int c, float r) {
-        const float own = src[base + c] * r * wt[base + c];
+    // coordinate c of a head of the normed vector that starts at column `first` (weights wt), turned if it lies among
+    // the turning ones
+    auto turned = [&](int first, const float* wt, int base, int c, float r) {
+        const float own = val(first + base + c) * r * wt[base + c];
         if (c >= 2 * half) return own;
-        const int mate = c ^ 1;
-        const float other = src[base + mate] * r * wt[base + mate];
-        const float co = cr[c >> 1], si = sr[c >> 1];
-        return (c & 1) ? own * co + other * si : own * co - other * si;
+        const int mate = split_half ? (c < half ? c + half : c - half) : c ^ 1;
+        const bool second = split_half ? c >= half : (c & 1);
+        const int pair = split_half ? (c < half ? c : c - half) : c >> 1;
+        const float other = val(first + base + mate) * r * wt[base + mate];
+        const float co = cr[pair], si = sr[pair];
+        return second ? own * co + other * si : own * co - other * si;
     };
     for (int i = threadIdx.x; i < heads * pad; i += 256) {
         const int h = i / pad, c = i % pad;
-        store_f32(q_out + row * (size_t)(heads * pad) + i, c < dim ? turned(pr, qw, h * dim, c, rq) : 0.f);
+        store_f32(q_out + row * (size_t)(heads * pad) + i, c < dim ? turned(0, qw, h * dim, c, rq) : 0.f);
     }
     if (!has_kv) return;
     const int slot = slots[row];
@@ -168,25 +186,27 @@ whole_norm_rope_scatter_kernel(const float* __restrict__ proj, int ld, const flo
     const size_t page = slot / page_size, off = slot % page_size;
     for (int i = threadIdx.x; i < kv_heads * pad; i += 256) {
         const int h = i / pad, c = i % pad;
-        const float kv = c < dim ? turned(pr + nq, kw, h * dim, c, rk) : 0.f;
-        const float vv = c < vdim ? pr[nq + nk + h * vdim + c] : 0.f;
+        const float kv = c < dim ? turned(nq, kw, h * dim, c, rk) : 0.f;
+        const float vv = c < vdim ? val(nq + nk + h * vdim + c) * (value_norm ? rv[h] : 1.0f) : 0.f;
         store_f32(kcache + ((page * kv_heads + h) * page_size + off) * pad + c, kv);
         store_f32(vcache + ((page * kv_heads + h) * pad + c) * page_size + off, vv);
     }
 }
 
-extern "C" int cisr_whole_norm_rope_scatter(const float* proj, int ld, const float* qw, const float* kw, const int* positions,
-                                            const int* slots, const float* cosines, const float* sines, int half, int max_pos,
-                                            void* q_out, void* kcache, void* vcache, int rows, int heads, int kv_heads, int dim,
-                                            int vdim, int pad, int page_size, float eps, int has_kv, int dtype, hipStream_t stream) {
+extern "C" int cisr_whole_norm_rope_scatter(const float* proj, int ld, const float* bias, const float* qw, const float* kw,
+                                            const int* positions, const int* slots, const float* cosines, const float* sines, int half,
+                                            int max_pos, void* q_out, void* kcache, void* vcache, int rows, int heads, int kv_heads,
+                                            int dim, int vdim, int pad, int page_size, float eps, int has_kv, int split_half,
+                                            int value_norm, int dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (dim <= 0 || dim > pad || vdim > pad || 2 * half > dim || half < 0 || heads <= 0 || (has_kv && (kv_heads <= 0 || page_size <= 0)))
+    if (dim <= 0 || dim > pad || vdim > pad || 2 * half > dim || half < 0 || heads <= 0 || (has_kv && (kv_heads <= 0 || page_size <= 0)) ||
+        (value_norm && kv_heads > WN_MAX_KV_HEADS))
         return (int)hipErrorInvalidValue;
     if (dtype == DT_F32)
-        whole_norm_rope_scatter_kernel<float><<<rows, 256, 0, stream>>>(proj, ld, qw, kw, positions, slots, cosines, sines, half, max_pos,
-            (float*)q_out, (float*)kcache, (float*)vcache, heads, kv_heads, dim, vdim, pad, page_size, eps, has_kv);
+        whole_norm_rope_scatter_kernel<float><<<rows, 256, 0, stream>>>(proj, ld, bias, qw, kw, positions, slots, cosines, sines, half, max_pos,
+            (float*)q_out, (float*)kcache, (float*)vcache, heads, kv_heads, dim, vdim, pad, page_size, eps, has_kv, split_half, value_norm);
     else
-        whole_norm_rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, ld, qw, kw, positions, slots, cosines, sines, half, max_pos,
-            (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, vdim, pad, page_size, eps, has_kv);
+        whole_norm_rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, ld, bias, qw, kw, positions, slots, cosines, sines, half, max_pos,
+            (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, vdim, pad, page_size, eps, has_kv, split_half, value_norm);
     return CISR_LAUNCH_CHECK();
 }

@@ -96,6 +96,104 @@ extern "C" int cisr_experts_route(const float* logits, int ld, const float* bias
     return CISR_LAUNCH_CHECK();
 }
 
+// Routing by scores: s = softmax of the logits over all `outputs` of the router; the choice goes by s + correction
+// (null: by s), held to the `keep` groups, of `groups` equal groups of neighbours, whose largest choice score is
+// largest (groups 0: no groups); the `top` largest are chosen (the lowest index wins a tie) and weigh s itself, not
+// normed again.  A thread a row; float arithmetic.
+__global__ void __launch_bounds__(256)
+route_scored_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int* __restrict__ chosen,
+                    float* __restrict__ weights, int rows, int outputs, int top, int groups, int keep) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= rows) return;
+    const float* lr = logits + (size_t)row * ld;
+    float largest = -INFINITY, den = 0.f;
+    for (int e = 0; e < outputs; ++e) largest = fmaxf(largest, lr[e]);
+    for (int e = 0; e < outputs; ++e) den += expf(lr[e] - largest);
+    auto score = [&](int e) { return expf(lr[e] - largest) / den; };
+    auto choice = [&](int e) { return score(e) + (correction ? correction[e] : 0.f); };
+    unsigned long long kept = ~0ull;                       // groups that may be chosen from (at most 64 groups)
+    const int per = groups > 0 ? outputs / groups : outputs;
+    if (groups > 0) {
+        kept = 0ull;
+        for (int k = 0; k < keep; ++k) {
+            int best = -1;
+            float bv = -INFINITY;
+            for (int g = 0; g < groups; ++g) {
+                if ((kept >> g) & 1ull) continue;
+                float gv = -INFINITY;
+                for (int e = g * per; e < (g + 1) * per; ++e) gv = fmaxf(gv, choice(e));
+                if (best < 0 || gv > bv) { best = g; bv = gv; }
+            }
+            kept |= 1ull << best;
+        }
+    }
+    int ids[MAX_TOP];
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bv = -INFINITY;
+        for (int e = 0; e < outputs; ++e) {
+            if (groups > 0 && !((kept >> (e / per)) & 1ull)) continue;
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= ids[j] == e;
+            if (taken) continue;
+            const float v = choice(e);
+            if (best < 0 || v > bv) { best = e; bv = v; }
+        }
+        ids[k] = best;
+        chosen[(size_t)row * top + k] = best;
+        weights[(size_t)row * top + k] = score(best);
+    }
+}
+
+// `experts` of the router's `outputs` have matrices (the first ones): only their pairs are arranged into tiles.
+extern "C" int cisr_experts_route_scored(const float* logits, int ld, const float* correction, int* chosen, float* weights, int rows,
+                                         int outputs, int experts, int top, int groups, int keep, int max_tiles, int* pair_of_pos,
+                                         int* tile_expert, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    const bool arrange = pair_of_pos != nullptr;
+    if (outputs <= 0 || experts <= 0 || experts > outputs || top <= 0 || top > MAX_TOP || top > outputs || experts > 4096 || groups < 0 ||
+        groups > 64 || (groups > 0 && (outputs % groups || keep <= 0 || keep > groups || keep * (outputs / groups) < top)) ||
+        (arrange && (!tile_expert || (long long)max_tiles * EX_TILE < (long long)rows * top + (long long)experts * (EX_TILE - 1))))
+        return (int)hipErrorInvalidValue;
+    route_scored_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(logits, ld, correction, chosen, weights, rows, outputs, top, groups, keep);
+    int err = CISR_LAUNCH_CHECK();
+    if (err || !arrange) return err;
+    arrange_kernel<<<1, 1024, 3 * experts * sizeof(int), stream>>>(chosen, rows * top, experts, max_tiles, pair_of_pos, tile_expert);
+    return CISR_LAUNCH_CHECK();
+}
+
+// y[row] = sum_k weights[row, k] * (chosen[row, k] < experts ? down[row top + k] : x[row]) + shared[row]: the weighted sum
+// over a row's choices, a choice without matrices being the sublayer's input itself (x, in the activations' type), plus
+// what every row goes through.
+template <typename TX>
+__global__ void __launch_bounds__(256)
+experts_combine_kernel(const float* __restrict__ down, const float* __restrict__ weights, const int* __restrict__ chosen,
+                       const TX* __restrict__ x, const float* __restrict__ shared, float* __restrict__ y, int dim, int top,
+                       int experts) {
+    const size_t row = blockIdx.x;
+    float w[MAX_TOP];
+    int real[MAX_TOP];
+    for (int k = 0; k < top; ++k) {
+        w[k] = weights[row * top + k];
+        const int e = chosen[row * top + k];
+        real[k] = e >= 0 && e < experts;
+    }
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        float v = shared ? shared[row * dim + d] : 0.f;
+        for (int k = 0; k < top; ++k) v += w[k] * (real[k] ? down[(row * top + k) * dim + d] : load_f32(x + row * dim + d));
+        y[row * dim + d] = v;
+    }
+}
+
+extern "C" int cisr_experts_combine(const float* down, const float* weights, const int* chosen, const void* x, int x_dtype,
+                                    const float* shared, float* y, int rows, int dim, int top, int experts, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim <= 0 || top <= 0 || top > MAX_TOP || experts < 0) return (int)hipErrorInvalidValue;
+    if (x_dtype == DT_F32) experts_combine_kernel<float><<<rows, 256, 0, stream>>>(down, weights, chosen, (const float*)x, shared, y, dim, top, experts);
+    else experts_combine_kernel<bf16_t><<<rows, 256, 0, stream>>>(down, weights, chosen, (const bf16_t*)x, shared, y, dim, top, experts);
+    return CISR_LAUNCH_CHECK();
+}
+
 // relu(z)^2, the experts' activation; ACT 0: none
 template <int ACT>
 __device__ __forceinline__ float expert_act(float v) {
@@ -311,9 +409,10 @@ expert_gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
 template <typename TC, int ACT>
 __global__ void __launch_bounds__(256)
 expert_rows_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const int* __restrict__ chosen,
-                   int gather_div, TC* __restrict__ C, int ldc, int N, int K) {
+                   int gather_div, TC* __restrict__ C, int ldc, int N, int K, int experts) {
     const int pair = blockIdx.y;
     const int e = chosen[pair];
+    if (e < 0 || e >= experts) return;                       // (a choice without matrices: its row is left alone)
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const int n_first = (blockIdx.x * 4 + wave) * 4;
     if (n_first >= N) return;
@@ -360,18 +459,18 @@ extern "C" int cisr_experts_rows_ok(int K, int lda, int pairs) {
 }
 
 extern "C" int cisr_experts_rows(const void* A, int lda, const void* W, const int* chosen, int gather_div, void* C, int ldc,
-                                 int pairs, int N, int K, int act, int out_dtype, hipStream_t stream) {
+                                 int pairs, int N, int K, int act, int out_dtype, int experts, hipStream_t stream) {
     if (pairs <= 0 || N <= 0) return 0;
     if (!cisr_experts_rows_ok(K, lda, pairs) || ((uintptr_t)A) % 16 || ((uintptr_t)W) % 16) return (int)hipErrorInvalidValue;
     const dim3 grid((N + 15) / 16, pairs);
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
     if (out_dtype == DT_F32) {
-        if (act) expert_rows_kernel<float, 1><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (float*)C, ldc, N, K);
-        else expert_rows_kernel<float, 0><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (float*)C, ldc, N, K);
+        if (act) expert_rows_kernel<float, 1><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (float*)C, ldc, N, K, experts);
+        else expert_rows_kernel<float, 0><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (float*)C, ldc, N, K, experts);
     } else {
-        if (act) expert_rows_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (bf16_t*)C, ldc, N, K);
-        else expert_rows_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (bf16_t*)C, ldc, N, K);
+        if (act) expert_rows_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (bf16_t*)C, ldc, N, K, experts);
+        else expert_rows_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>(a, lda, w, chosen, gather_div, (bf16_t*)C, ldc, N, K, experts);
     }
     return CISR_LAUNCH_CHECK();
 }

@@ -442,12 +442,12 @@ extern "C" int cisr_gemm_bf16_heads(const void* A, int lda, int a_head, const vo
     return (int)hipErrorInvalidValue;
 }
 
-// C = act(A . W^T) with an ungated activation (ACT_GELU, ACT_GELU_TANH) as the epilogue; the tile is picked as for the
+// C = act(A . W^T) with an ungated activation (ACT_GELU, ACT_GELU_TANH, ACT_RELU2) as the epilogue; the tile is picked as for the
 // plain product.
 extern "C" int cisr_gemm_bf16_act(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
                                   int out_dtype, int act, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K <= 0 || (act != ACT_GELU && act != ACT_GELU_TANH)) return (int)hipErrorInvalidValue;
+    if (K <= 0 || act < ACT_GELU || act > ACT_RELU2) return (int)hipErrorInvalidValue;
     const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
     const HeadBatch batch{0, 0, 0, nullptr, 0, act};
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };

@@ -73,7 +73,7 @@ extern "C" int cisr_gemm_skinny_bf16(const void* A, int lda, const void* W, int 
     return skinny_entry(A, lda, W, ldw, C, ldc, R, ldr, M, N, K, out_dtype, dual_off, norm_w, eps, rows, GateLaw{}, stream, ACT_NONE);
 }
 
-// C = act(A . W^T): the same product with an ungated activation (ACT_GELU, ACT_GELU_TANH) before the store.
+// C = act(A . W^T): the same product with an ungated activation (ACT_GELU, ACT_GELU_TANH, ACT_RELU2) before the store.
 extern "C" int cisr_gemm_skinny_bf16_act(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
                                          int out_dtype, int act, hipStream_t stream) {
     return skinny_entry(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, out_dtype, 0, nullptr, 0.f, nullptr, GateLaw{}, stream, act);
@@ -91,7 +91,7 @@ static int skinny_entry(const void* A, int lda, const void* W, int ldw, void* C,
                         int ldr, int M, int N, int K, int out_dtype, int dual_off, const float* norm_w,
                         float eps, const int* rows, GateLaw law, hipStream_t stream, int act) {
     if (M <= 0 || N <= 0) return 0;
-    if (act < ACT_NONE || act > ACT_GELU_TANH || (act && (R || dual_off > 0))) return (int)hipErrorInvalidValue;
+    if (act < ACT_NONE || act > ACT_RELU2 || (act && (R || dual_off > 0))) return (int)hipErrorInvalidValue;
     if (M > 64 || K <= 0 || K % 8 || lda % 8 || ldw % 8 || !aligned16(A) || !aligned16(W) ||
         (R && out_dtype != DT_F32) || (norm_w && !aligned16(norm_w)) || (dual_off > 0 && (R || out_dtype != DT_BF16)))
         return (int)hipErrorInvalidValue;

@@ -369,3 +369,15 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
                        block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles, key_groups=halves,
                        head_bias=head_bias)
     return None
+
+
+def talking_attention(ctx, q, kcache, vcache, view, out, heads, kv_heads, vdim, pad, mix, scale, temp=None, sink=None,
+                      window=None, chunk=None, gate=None):
+    """out[r] = attention of row r over its request's cached keys where the scores of all heads of a row are mixed
+    (`mix` [heads, heads], after `temp`[g] scale) before the softmax, whose denominator holds exp(`sink`[h]) as well; a
+    row sees its block of `chunk` positions up to itself (or the last `window` keys, or all); `gate`: the result times
+    sigmoid(gate) element by element.  The mix needs every head's score of a (row, key) pair in one place, so this is a
+    kernel of its own beside the paged attention above: one block a row walks the row's keys for all heads."""
+    ops.attention_talking(q, q.stride(0), kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out, heads, kv_heads, vdim, pad,
+                          view.page_size, mix, scale, temp=temp, sink=sink, window=window, chunk=chunk, gate=gate)
+    return out

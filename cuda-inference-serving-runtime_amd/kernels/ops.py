@@ -69,7 +69,7 @@ def _declare(h):
         "cisr_gemm_skinny_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
         "cisr_gemm_wide_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p, C.c_longlong, p],
         "cisr_gemm_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
-        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, i, i, p],
+        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, i, i, f, f, p],
         "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
         "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
         "cisr_head_gate": [p, p, i, p, i, i, i, i, i, p],
@@ -85,10 +85,14 @@ def _declare(h):
         "cisr_attn_merge_sum": [p, p, i, i, i, i, p, p],
         "cisr_embedding_pairs": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, f, i, ll, ll, i, i, i, p],
         "cisr_gate_post_norm": [p, p, i, p, p, i, p, p, p, i, i, f, f, i, p],
-        "cisr_whole_norm_rope_scatter": [p, i, p, p, p, p, p, p, i, i, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
+        "cisr_whole_norm_rope_scatter": [p, i, p, p, p, p, p, p, p, i, i, p, p, p, i, i, i, i, i, i, i, f, i, i, i, i, p],
+        "cisr_attn_talking": [p, i, p, p, p, p, p, p, p, p, p, i, p, i, i, i, i, i, i, i, i, i, f, i, p],
         "cisr_experts_route": [p, i, p, p, p, i, i, i, i, p, p, p],
         "cisr_experts_gemm": [p, i, p, p, p, i, i, p, i, i, i, i, i, i, i, p],
-        "cisr_experts_rows": [p, i, p, p, i, p, i, i, i, i, i, i, p],
+        "cisr_experts_rows": [p, i, p, p, i, p, i, i, i, i, i, i, i, p],
+        "cisr_experts_route_scored": [p, i, p, p, p, i, i, i, i, i, i, i, p, p, p],
+        "cisr_experts_combine": [p, p, p, p, i, p, p, i, i, i, i, p],
+        "cisr_bias_act": [p, p, p, ll, i, i, i, p],
         "cisr_experts_rows_ok": [i, i, i],
     }
     for name, args in sig.items():
@@ -366,6 +370,35 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
 LIBRARY_MIN_ROWS = 65
 LIBRARY_MIN_BYTES = 8 << 20
 LIBRARY_GATED_MIN_ROWS, LIBRARY_GATED_MIN_BYTES = 33, 64 << 20
+
+
+def attention_talking(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, vdim, pad, page_size,
+                      mix, scale, temp=None, sink=None, window=None, chunk=None, gate=None):
+    """Attention whose scores are mixed over the heads before the softmax: s_h = sum_g mix[h, g] temp[g] scale (q_g . k),
+    weights exp(s_h) / (exp(sink_h) + sum over the visible keys), out_h = sum w_h v of the head's key/value head, times
+    sigmoid(gate) element by element.  A row at position p sees the keys of its block of `chunk` positions up to itself
+    (or the last `window`, or all).  q [T, >= heads * pad] and the pages hold heads of `pad` coordinates, the rest zero;
+    out [T, heads * vdim]; mix float [heads, heads], temp and sink float [heads] or None; gate a float view
+    [T, heads * vdim] or None."""
+    rows = out.shape[0]
+    pages = kcache.shape[0]
+    gp, ldg = None, 0
+    if gate is not None:
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (rows, heads * vdim) or gate.stride(1) != 1 or not gate.is_cuda:
+            raise KernelError("attention_talking: the gate must be float [T, heads * vdim] with unit stride")
+        gp, ldg = gate.data_ptr(), gate.stride(0)
+    if q.dim() != 2 or q.shape[0] != rows or q.stride(1) != 1 or q.shape[1] < heads * pad or q.dtype != out.dtype or not q.is_cuda:
+        raise KernelError("attention_talking: q must be [T, >= heads * pad] of the output's dtype")
+    width = tables.shape[1]
+    _check(lib().cisr_attn_talking(q.data_ptr(), int(q_row_stride), _dev(kcache, "kcache", out.dtype, (pages, kv_heads, page_size, pad)),
+                                   _dev(vcache, "vcache", out.dtype, (pages, kv_heads, pad, page_size)),
+                                   _dev(tables, "tables", torch.int32), _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
+                                   _dev(positions, "positions", torch.int32, (rows,)), _dev(mix, "mix", torch.float32, (heads, heads)),
+                                   None if temp is None else _dev(temp, "temp", torch.float32, (heads,)),
+                                   None if sink is None else _dev(sink, "sink", torch.float32, (heads,)), gp, ldg,
+                                   _dev(out, "out", None, (rows, heads * vdim)), rows, heads, kv_heads, vdim, pad, page_size, width,
+                                   int(window or 0), int(chunk or 0), float(scale), _storage(out, "out"), _stream()), "attention_talking")
+    return out
 
 
 class ScratchPool:
@@ -924,9 +957,11 @@ def gemm_for_norm(a, w, out, make_buffer, scratch=None):
 
 def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
     """x += mult * rmsnorm(y) * weight, in place (all float, [T, H]).  With `second` = (y2, w1, w2) the row that is
-    normed is (rmsnorm(y) w1 + rmsnorm(y2) w2) / 2: two sublayers side by side.  `weight` None: no outer norm,
+    normed is (rmsnorm(y) w1 + rmsnorm(y2) w2) / 2: two sublayers side by side; with `second` = (y2, c1, c2), two
+    numbers, it is the plain sum c1 y + c2 y2.  `weight` None: no outer norm,
     x += mult * row.  `following` = (weight float [H], eps, out [T, H] float or bf16): the norm that reads x next is made
-    by the same kernel, out = rmsnorm(x) * weight.  y (and y2) may be a Partials of [T, H]: its slices are added on the way."""
+    by the same kernel, out = rmsnorm(x) * weight; a weight of None: out is the new x itself in out's type.
+    y (and y2) may be a Partials of [T, H]: its slices are added on the way."""
     rows, dim = x.shape
     xp = _dev(x, "x", torch.float32)
 
@@ -941,16 +976,21 @@ def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
     slices_b = 0
     wp = None if weight is None else _dev(weight, "weight", torch.float32, (dim,))
     ap = bp = w2p = None
+    ca = cb = 0.0
     if second is not None:
         y2, w1, w2 = second
         bp, slices_b = operand(y2, "y2")
-        ap, w2p = _dev(w1, "w1", torch.float32, (dim,)), _dev(w2, "w2", torch.float32, (dim,))
+        if isinstance(w1, torch.Tensor):
+            ap, w2p = _dev(w1, "w1", torch.float32, (dim,)), _dev(w2, "w2", torch.float32, (dim,))
+        else:
+            ca, cb = float(w1), float(w2)
     np_, neps, op, odt = None, 0.0, None, F32
     if following is not None:
         nw, neps, out = following
-        np_, op, odt = _dev(nw, "following weight", torch.float32, (dim,)), _dev(out, "following out", None, (rows, dim)), _storage(out, "following out")
+        np_ = None if nw is None else _dev(nw, "following weight", torch.float32, (dim,))
+        op, odt = _dev(out, "following out", None, (rows, dim)), _storage(out, "following out")
     _check(lib().cisr_post_norm_add(xp, yp, ap, bp, w2p, wp, rows, dim, float(eps), float(mult), np_, float(neps), op, odt,
-                                    slices_a, slices_b, _stream()), "post_norm_add")
+                                    slices_a, slices_b, ca, cb, _stream()), "post_norm_add")
     return x
 
 
@@ -1079,7 +1119,7 @@ def heads_product(a, a_head, w, out, out_head, gate=None):
     return out
 
 
-GELU_KINDS = {"gelu": 0, "gelu_erf": 0, "gelu_tanh": 1}
+GELU_KINDS = {"gelu": 0, "gelu_erf": 0, "gelu_tanh": 1, "relu2": 2}      # ungated activations (relu2: relu(z)^2)
 
 
 def gemm_gelu(a, w, out, kind="gelu", scratch=None, product=None):
@@ -1105,6 +1145,15 @@ def gemm_gelu(a, w, out, kind="gelu", scratch=None, product=None):
     if product is None:
         raise KernelError("gemm_gelu: this product needs a buffer for its result before the activation")
     return gelu(gemm(a, w, product, scratch=scratch), out, kind)
+
+
+def bias_act(x, bias, out, kind):
+    """out = act(x + bias[column]): the activation of a product with a bias (float [N]); x, out [M, N] of one dtype."""
+    if kind not in GELU_KINDS:
+        raise KernelError(f"bias_act: unknown activation {kind!r}")
+    _check(lib().cisr_bias_act(_dev(x, "x"), _dev(bias, "bias", torch.float32, (x.shape[1],)), _dev(out, "out", x.dtype, x.shape), x.numel(),
+                               x.shape[1], GELU_KINDS[kind], _storage(x, "x"), _stream()), "bias_act")
+    return out
 
 
 def gelu(x, out, kind="gelu"):
@@ -1135,6 +1184,8 @@ def _rec():
             "cisr_delta_scan": [p, i, p, i, p, i, p, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
             "cisr_unit_heads": [p, i, i, i, i, i, f, f, p],
             "cisr_mingru_scan": [p, i, p, p, p, i, p, p, p, i, i, i, i, p, i, i, p],
+            "cisr_mlstm_gates": [p, i, p, i, p, p, p, i, p, p, p, p, p, ll, p, p, i, i, i, f, p],
+            "cisr_mlstm_finish": [p, p, p, i, p, p, i, i, i, f, f, i, p],
         }
         for name, args in sig.items():
             fn = getattr(h, name)
@@ -1418,14 +1469,17 @@ def gate_post_norm(x, y, weight, eps, alpha, gate=None, gate_bias=None, cast=Non
 
 
 def whole_norm_rope_scatter(proj, q_norm, k_norm, positions, slots, cos, sin, q_out, kcache, vcache, heads, kv_heads, dim, vdim,
-                            pad, page_size, eps):
+                            pad, page_size, eps, bias=None, split_half=False, value_norm=False):
     """Rows of a projection with float results [q: heads x dim | k: kv_heads x dim | v: kv_heads x vdim | ...]: q and k
     RMS-normed over all their heads at once (weights float [heads * dim], [kv_heads * dim]), the first 2 * cos.shape[1]
     coordinates of every head turned in neighbouring pairs by the position (cos / sin float [max_pos, pairs]), q into
     q_out [T, heads * pad], k and v into the pages at `slots` as heads of `pad` coordinates whose rest is zero.
-    kcache None: the rows have queries only (a layer that reads another's cache)."""
+    kcache None: the rows have queries only (a layer that reads another's cache).  `bias`: float over the q, k and v
+    columns, added before everything else; `split_half`: the pairs are (i, i + pairs) instead of neighbours;
+    `value_norm`: each head's value is divided by its root mean square over vdim (eps, no weight) before it is stored."""
     rows, ld = proj.shape
     has_kv = kcache is not None
+    bp = None if bias is None else _dev(bias, "bias", torch.float32, (heads * dim + (kv_heads * (dim + vdim) if has_kv else 0),))
     if proj.dtype != torch.float32 or proj.stride(1) != 1 or not proj.is_cuda:
         raise KernelError("whole_norm_rope_scatter: a float projection with contiguous rows")
     if dim > pad or vdim > pad or ld < heads * dim + (kv_heads * (dim + vdim) if has_kv else 0):
@@ -1440,12 +1494,12 @@ def whole_norm_rope_scatter(proj, q_norm, k_norm, positions, slots, cos, sin, q_
         vp = _dev(vcache, "vcache", q_out.dtype, (pages, kv_heads, pad, page_size))
         sp = _dev(slots, "slots", torch.int32, (rows,))
         kw = _dev(k_norm, "k_norm", torch.float32, (kv_heads * dim,))
-    _check(lib().cisr_whole_norm_rope_scatter(proj.data_ptr(), proj.stride(0), _dev(q_norm, "q_norm", torch.float32, (heads * dim,)), kw,
+    _check(lib().cisr_whole_norm_rope_scatter(proj.data_ptr(), proj.stride(0), bp, _dev(q_norm, "q_norm", torch.float32, (heads * dim,)), kw,
                                               _dev(positions, "positions", torch.int32, (rows,)), sp,
                                               _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, half)),
                                               half, max_pos, _dev(q_out, "q_out", None, (rows, heads * pad)), kp, vp, rows, heads,
-                                              kv_heads, dim, vdim, pad, page_size, float(eps), int(has_kv), _storage(q_out, "q_out"),
-                                              _stream()), "whole_norm_rope_scatter")
+                                              kv_heads, dim, vdim, pad, page_size, float(eps), int(has_kv), int(bool(split_half)),
+                                              int(bool(value_norm)), _storage(q_out, "q_out"), _stream()), "whole_norm_rope_scatter")
     return q_out
 
 
@@ -1481,6 +1535,44 @@ def experts_route(logits, bias, top, chosen, weights, pair_of_pos=None, tile_exp
     return chosen, weights
 
 
+def experts_route_scored(logits, correction, top, chosen, weights, experts, groups=None, pair_of_pos=None, tile_expert=None):
+    """Routing by scores: logits a float view [T, outputs]; s = softmax over all outputs; the choice goes by s + correction
+    (float [outputs] or None), held to the best `groups[1]` of `groups[0]` equal groups of neighbours (a group's score is
+    its largest choice score); chosen int32 [T, top] (the lowest index wins a tie), weights float [T, top] = s of the
+    chosen, not normed again.  The first `experts` outputs have matrices: only their pairs are ordered by expert into
+    pair_of_pos / tile_expert (as experts_route does), the others are left to the caller."""
+    rows, outputs = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1 or not logits.is_cuda:
+        raise KernelError("experts_route_scored: float logits with contiguous rows")
+    count, keep = groups or (0, 0)
+    if not 0 < top <= min(outputs, 16) or not 0 < experts <= outputs or count > 64:
+        raise KernelError(f"experts_route_scored: {top} of {outputs} outputs, {experts} with matrices, {count} groups")
+    tiles, pp, tp = 0, None, None
+    if pair_of_pos is not None:
+        tiles = tile_expert.shape[0]
+        if tiles < expert_tiles(rows, top, experts):
+            raise KernelError(f"experts_route_scored: {tiles} tiles for {rows} rows x {top} of {experts} experts")
+        pp, tp = _dev(pair_of_pos, "pair_of_pos", torch.int32, (tiles * EXPERT_TILE,)), _dev(tile_expert, "tile_expert", torch.int32, (tiles,))
+    _check(lib().cisr_experts_route_scored(logits.data_ptr(), logits.stride(0),
+                                           None if correction is None else _dev(correction, "correction", torch.float32, (outputs,)),
+                                           _dev(chosen, "chosen", torch.int32, (rows, top)), _dev(weights, "weights", torch.float32, (rows, top)),
+                                           rows, outputs, int(experts), top, int(count), int(keep), tiles, pp, tp, _stream()), "experts_route_scored")
+    return chosen, weights
+
+
+def experts_combine(down, weights, chosen, x, y, experts, shared=None):
+    """y[r] = sum_k weights[r, k] * (down[r * top + k] if chosen[r, k] < experts else x[r]) + shared[r]: the weighted sum
+    over a row's choices (a choice without matrices is the input x itself) plus the rows every token goes through.
+    down [T * top, H], shared and y [T, H] are float, x [T, H] float or bf16."""
+    rows, top = weights.shape
+    dim = y.shape[1]
+    _check(lib().cisr_experts_combine(_dev(down, "down", torch.float32, (rows * top, dim)), _dev(weights, "weights", torch.float32),
+                                      _dev(chosen, "chosen", torch.int32, (rows, top)), _dev(x, "x", None, (rows, dim)), _storage(x, "x"),
+                                      None if shared is None else _dev(shared, "shared", torch.float32, (rows, dim)),
+                                      _dev(y, "y", torch.float32, (rows, dim)), rows, dim, top, int(experts), _stream()), "experts_combine")
+    return y
+
+
 EXPERT_ROWS_PAIRS = 32     # steps of at most this many (row, choice) pairs stream each pair's matrices (experts_rows)
 
 
@@ -1501,7 +1593,7 @@ def experts_rows(a, w, chosen, out, top=0, act=False):
     if a.shape[0] < (-(-pairs // top) if top > 0 else pairs):
         raise KernelError("experts_rows: too few operand rows")
     _check(lib().cisr_experts_rows(a.data_ptr(), a.stride(0), _dev(w, "w"), _dev(chosen, "chosen", torch.int32), int(top), _dev(out, "out"),
-                                   out.stride(0), pairs, n, k, int(bool(act)), _storage(out, "out"), _stream()), "experts_rows")
+                                   out.stride(0), pairs, n, k, int(bool(act)), _storage(out, "out"), int(experts), _stream()), "experts_rows")
     return out
 
 
@@ -1524,6 +1616,39 @@ def experts_gemm(a, w, pair_of_pos, tile_expert, out, top=0, scatter=False, act=
                                    _dev(tile_expert, "tile_expert", torch.int32), _dev(pair_of_pos, "pair_of_pos", torch.int32),
                                    int(top), int(bool(scatter)), _dev(out, "out"), out.stride(0), tiles, n, k, int(bool(act)),
                                    _storage(a, "a"), _storage(out, "out"), _stream()), "experts_gemm")
+    return out
+
+
+def mlstm_gates(zi, zf, bias_i, bias_f, v, decay, step, top, vx, top_state, seg_start, state_slots, heads, vdim, cap):
+    """The operands of the matrix memory's scan from the projections' float results: log gates i = cap tanh((zi + bi) /
+    cap), f = logsigmoid(cap tanh((zf + bf) / cap)) (zi, zf float views [T, heads]); along every segment's rows the
+    running maximum m' = max(f + m, i), from `top_state`[slot, head] and back into it; decay = exp(f + m - m'), step =
+    exp(i - m') and top = m', float [T, heads]; vx [T, heads * (vdim + 1)] = the values v (a float view [T, heads *
+    vdim]) with a column of ones a head."""
+    T = v.shape[0]
+    segments = state_slots.shape[0]
+    ip, ldi = _rows_of(zi, "zi", heads)
+    fp, ldf = _rows_of(zf, "zf", heads)
+    vp, ldv = _rows_of(v, "v", heads * vdim)
+    if top_state.dtype != torch.float32 or top_state.dim() != 2 or top_state.stride(1) != 1 or top_state.shape[1] < heads or not top_state.is_cuda:
+        raise KernelError("mlstm_gates: the running maxima are float [slots, >= heads]")
+    _check(_rec().cisr_mlstm_gates(ip, ldi, fp, ldf, _dev(bias_i, "bias_i", torch.float32, (heads,)), _dev(bias_f, "bias_f", torch.float32, (heads,)),
+                                   vp, ldv, _dev(decay, "decay", torch.float32, (T, heads)), _dev(step, "step", torch.float32, (T, heads)),
+                                   _dev(top, "top", torch.float32, (T, heads)), _dev(vx, "vx", torch.float32, (T, heads * (vdim + 1))),
+                                   top_state.data_ptr(), top_state.stride(0), _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
+                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, vdim, float(cap), _stream()),
+           "mlstm_gates")
+
+
+def mlstm_finish(o, top, gate, weight, out, heads, vdim, eps, floor=1e-6):
+    """The matrix memory's result from its scan's: o float [T, heads * (vdim + 1)], the last column of a head n . q;
+    out[t, h] = rms(o_h / (max(|n . q|, exp(-top)) + floor)) * weight * sigmoid(gate), rms over vdim with eps; gate a
+    float view [T, heads * vdim], weight float [heads * vdim], out [T, heads * vdim] float or bf16."""
+    T = o.shape[0]
+    gp, ldg = _rows_of(gate, "gate", heads * vdim)
+    _check(_rec().cisr_mlstm_finish(_dev(o, "o", torch.float32, (T, heads * (vdim + 1))), _dev(top, "top", torch.float32, (T, heads)), gp, ldg,
+                                    _dev(weight, "weight", torch.float32, (heads * vdim,)), _dev(out, "out", None, (T, heads * vdim)),
+                                    T, heads, vdim, float(eps), float(floor), _storage(out, "out"), _stream()), "mlstm_finish")
     return out
 
 

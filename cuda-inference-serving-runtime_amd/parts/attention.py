@@ -17,7 +17,7 @@ import math
 
 import torch
 
-from ..cache.pages import KVNeed
+from ..cache.pages import ChunkNeed, KVNeed
 from ..kernels import attention as kernel, ops
 from .base import Mixer, TensorSpec, matrix_operand, register_part
 
@@ -435,6 +435,112 @@ class SigmoidAttention(Mixer):
         return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
+class TalkingAttention(Mixer):
+    """Grouped-query softmax attention over the paged cache whose scores are mixed over the heads before the softmax:
+    s_h = sum_g `talk`[h, g] (`temp`[g] scale q_g . k), a learned number a head (`sink`) in every softmax's denominator
+    (a key without a value), and the heads' results gated element by element by sigmoid(W_g h) before the output
+    projection.  Queries and keys are RMS-normed over the whole projection (all heads at once, a weight an element)
+    before `position` turns the first `position.rotary_dim` coordinates of every head (split-half pairs); each head's
+    value is divided by its root mean square and cached so; keys and values may differ in size (`dim`, `vdim`);
+    projections have biases (`<tensor>.b`) where `bias` names them.  A row sees the keys of its own block of `chunk`
+    positions up to itself (blocks counted from position 0; None: all keys before it).
+
+    The pages hold heads of `pad` = max(dim, vdim) coordinates (rounded up to a multiple of 8), the rest zero; with a
+    `chunk` the cache keeps the last `chunk` keys (ChunkNeed: pages before a row's block go back).  The scores of all
+    heads of a row meet in one kernel (ops.attention_talking).  `names`: the tensors' names under `name`."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm", "talk": "talk",
+             "temp": "temp", "sink": "sink"}
+
+    def __init__(self, name, hidden, heads, kv_heads, dim, vdim, scale, eps, position, chunk=None, bias=("q", "k", "v", "o"),
+                 temp=True, sink=True, gate=True, value_norm=True, names=None):
+        if heads % kv_heads:
+            raise ValueError(f"{heads} query heads are not a multiple of {kv_heads} key/value heads")
+        self.pad = -(-max(dim, vdim) // 8) * 8
+        if not scale > 0:
+            raise ValueError("the score scale must be positive")
+        if getattr(position, "pairing", "split_half") != "split_half" or getattr(position, "rotary_dim", 0) > dim:
+            raise ValueError("the position part must turn split-half pairs of at most `dim` coordinates")
+        if chunk is not None and chunk <= 0:
+            raise ValueError("a block of positions holds at least one")
+        self.name, self.hidden, self.heads, self.kv_heads, self.dim, self.vdim = name, hidden, heads, kv_heads, dim, vdim
+        self.scale, self.eps, self.position, self.chunk = float(scale), float(eps), position, chunk
+        self.bias, self.has_temp, self.has_sink, self.has_gate, self.value_norm = tuple(bias), bool(temp), bool(sink), bool(gate), bool(value_norm)
+        self.names = {**self.NAMES, **(names or {})}
+        self.w_in = self.w_out = self.b_in = self.b_out = self.q_weight = self.k_weight = self.talk = self.temp = self.sink = None
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def cache_need(self):
+        return KVNeed(self.kv_heads, self.pad) if self.chunk is None else ChunkNeed(self.kv_heads, self.pad, self.chunk, self.chunk)
+
+    def tensor_specs(self):
+        H, nh, nkv, D, V = self.hidden, self.heads, self.kv_heads, self.dim, self.vdim
+        t = self._tensor
+        rows = {"q": nh * D, "k": nkv * D, "v": nkv * V, "o": H}
+        specs = [TensorSpec(t("q"), (nh * D, H)), TensorSpec(t("k"), (nkv * D, H)), TensorSpec(t("v"), (nkv * V, H)),
+                 TensorSpec(t("q_norm"), (nh * D,), init="one_plus_normal"), TensorSpec(t("k_norm"), (nkv * D,), init="one_plus_normal"),
+                 TensorSpec(t("talk"), (nh, nh)), TensorSpec(t("o"), (H, nh * V))]
+        specs += [TensorSpec(t(p) + ".b", (rows[p],)) for p in self.bias]
+        if self.has_temp:
+            specs.append(TensorSpec(t("temp"), (nh,), init="one_plus_normal"))
+        if self.has_sink:
+            specs.append(TensorSpec(t("sink"), (nh,)))
+        if self.has_gate:
+            specs.append(TensorSpec(t("g"), (nh * V, H)))
+        return specs
+
+    def bind(self, tensors, dtype):
+        t = self._tensor
+        inputs = ("q", "k", "v") + (("g",) if self.has_gate else ())
+        parts = [matrix_operand(tensors[t(p)], dtype) for p in inputs]
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:      # rows of the fused projection are a multiple of 8: zero rows at the end
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_out = matrix_operand(tensors[t("o")], dtype)
+
+        def f32(x):
+            return x.to(torch.float32).contiguous()
+        if any(p in self.bias for p in ("q", "k", "v")):
+            sizes = {"q": self.heads * self.dim, "k": self.kv_heads * self.dim, "v": self.kv_heads * self.vdim}
+            ref = parts[0]
+            self.b_in = torch.cat([f32(tensors[t(p) + ".b"]) if p in self.bias else torch.zeros(sizes[p], dtype=torch.float32, device=ref.device)
+                                   for p in ("q", "k", "v")]).contiguous()
+        self.b_out = f32(tensors[t("o") + ".b"]) if "o" in self.bias else None
+        self.q_weight, self.k_weight, self.talk = f32(tensors[t("q_norm")]), f32(tensors[t("k_norm")]), f32(tensors[t("talk")])
+        self.temp = f32(tensors[t("temp")]) if self.has_temp else None
+        self.sink = f32(tensors[t("sink")]) if self.has_sink else None
+
+    def prepare(self, device, dtype):
+        self.position.prepare(device, dtype)
+
+    def output(self, h, ctx, site, scale=1.0):
+        """The mixer's result times `scale`, float [T, hidden], without the residual sum."""
+        T = h.shape[0]
+        nh, nkv, D, V, pad = self.heads, self.kv_heads, self.dim, self.vdim, self.pad
+        gid, kcache, vcache = ctx.cache.pages_of_site(site)
+        view = ctx.kv[gid]
+        cos, sin = self.position.tables()
+        # queries, keys and values before their norms are float (the norms' statistics are), and so is the gate
+        proj = ops.gemm(h, self.w_in, ctx.buffer("tattn.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        q = ctx.buffer("tattn.q", (T, nh * pad), ctx.dtype)
+        ops.whole_norm_rope_scatter(proj, self.q_weight, self.k_weight, ctx.positions, view.slots, cos, sin, q, kcache, vcache,
+                                    nh, nkv, D, V, pad, view.page_size, self.eps, bias=self.b_in, split_half=True, value_norm=self.value_norm)
+        first = nh * D + nkv * (D + V)
+        act = ctx.buffer("tattn.act", (T, nh * V), ctx.dtype)
+        kernel.talking_attention(ctx, q, kcache, vcache, view, act, nh, nkv, V, pad, self.talk, self.scale, temp=self.temp, sink=self.sink,
+                                 chunk=self.chunk, gate=proj[:, first:first + nh * V] if self.has_gate else None)
+        y = ops.gemm(act, self.w_out, ctx.buffer("tattn.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+        return y if self.b_out is None else ops.bias_add(y, self.b_out)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
+
+
+register_part("mixer", "talking_attention", TalkingAttention)
 register_part("mixer", "attention", PagedAttention)
 register_part("mixer", "sigmoid_attention", SigmoidAttention)
 register_part("mixer", "latent_attention", LatentAttention)

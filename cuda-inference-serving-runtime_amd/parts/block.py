@@ -1,7 +1,8 @@
 """Arrangement of parts in a layer.  PreNormBlock is the Llama arrangement
 (reference: runtime/model.py:106-119): x = x + mixer(norm1(x)); x = x + ffn(norm2(x)),
 the residual stream x kept in float.  SandwichBlock norms each sublayer's result as well
-and scales it: x = x + m norm1b(mixer(norm1(x))); x = x + m norm2b(ffn(norm2(x))).  PostNormBlock norms after the
+and scales it: x = x + m norm1b(mixer(norm1(x))); x = x + m norm2b(ffn(norm2(x))); without the norms in front
+(`reads_stream`) its sublayers read x itself: x = x + m norm1b(mixer(x)).  PostNormBlock norms after the
 sum, and its sublayers read the stream itself: x = norm1(a x + g1 mixer(x)); x = norm2(a x + g2 ffn(x)), with
 optional gates g = sigmoid(W x + b) element by element."""
 import torch
@@ -86,12 +87,26 @@ class NormedMean:
         self.first, self.first_weight, self.second, self.second_weight, self.eps = first, first_weight, second, second_weight, eps
 
 
+class ScaledSum:
+    """What a mixer made of two mixers side by side may hand to the arrangement around it instead: a first + b second,
+    two float results [T, H] and two numbers.  The kernel that adds the sublayer's result makes the sum on the way."""
+
+    def __init__(self, first, first_scale, second, second_scale):
+        self.first, self.first_scale, self.second, self.second_scale = first, float(first_scale), second, float(second_scale)
+
+
 def add_sublayer(residual, result, norm, mult, eps=None, following=None):
-    """residual += mult * norm(result) (norm None: mult * result); `result` float rows or a NormedMean.
-    `following` = (norm part, out): the RMS norm that reads the residual stream next is made by the same kernel."""
+    """residual += mult * norm(result) (norm None: mult * result); `result` float rows, a NormedMean or a ScaledSum.
+    `following` = (norm part, out): the RMS norm that reads the residual stream next is made by the same kernel; with
+    CAST as the norm, `out` receives the new rows themselves in its type."""
     weight = None if norm is None else norm.weight
     eps = norm.eps if norm is not None else eps
-    then = None if following is None else (following[0].weight, following[0].eps, following[1])
+    then = None
+    if following is not None:
+        then = (None, 0.0, following[1]) if following[0] is CAST else (following[0].weight, following[0].eps, following[1])
+    if isinstance(result, ScaledSum):
+        return ops.post_norm_add(residual, result.first, weight, 0.0 if eps is None else eps, mult,
+                                 second=(result.second, result.first_scale, result.second_scale), following=then)
     if isinstance(result, NormedMean):
         if eps is not None and eps != result.eps:
             raise ValueError("the norms inside a mean of two results and the norm around it must share their eps (one kernel)")
@@ -104,10 +119,15 @@ class SandwichBlock(Part):
     """A norm before and after each sublayer, the normed result times `mult` added to the float residual stream.
     Its mixer and feed-forward give their result without the residual sum (`output`); `ffn` None: a layer without
     a feed-forward.  The norms after the sublayers are RMS norms (`weight`, `eps`); the sum, the norm and the scale
-    are one kernel."""
+    are one kernel.  `reads_stream`: there are no norms in front (`mixer_norm`, `ffn_norm` None) and the sublayers read
+    the residual stream itself, in the activations' type (that copy is made by the kernel that wrote the stream last)."""
 
-    def __init__(self, mixer_norm, mixer, mixer_post, ffn_norm=None, ffn=None, ffn_post=None, mult=1.0):
-        if (ffn is None) != (ffn_norm is None) or (ffn is None) != (ffn_post is None):
+    def __init__(self, mixer_norm, mixer, mixer_post, ffn_norm=None, ffn=None, ffn_post=None, mult=1.0, reads_stream=False):
+        self.reads_stream = bool(reads_stream)
+        if self.reads_stream:
+            if mixer_norm is not None or ffn_norm is not None or (ffn is None) != (ffn_post is None):
+                raise ValueError("sublayers that read the stream itself have no norm in front; a feed-forward comes with the norm after it")
+        elif (ffn is None) != (ffn_norm is None) or (ffn is None) != (ffn_post is None):
             raise ValueError("a feed-forward comes with the norms before and after it, or not at all")
         for post in (mixer_post, ffn_post):
             if post is not None and getattr(post, "fusable_as", None) != "rms":
@@ -148,13 +168,50 @@ class SandwichBlock(Part):
         return [a for p in self.parts() if hasattr(p, "step_arrays") for a in p.step_arrays()]
 
     def first_norm(self):
-        return self.mixer_norm
+        return CAST if self.reads_stream else self.mixer_norm
 
     @staticmethod
     def _plain_rms(norm):
         return norm is not None and getattr(norm, "fusable_as", None) == "rms"
 
+    def _forward_stream(self, residual, ctx, site):
+        """The layer whose sublayers read the stream itself: h is x in the activations' type (x itself in float32)."""
+        after = ctx.next_norm
+        ctx.next_norm = None
+        ctx.settle(residual)
+        narrow = ctx.dtype != torch.float32
+        T, H = residual.shape
+
+        def following(reader, tag):
+            # the copy of the new rows for whoever reads the stream next: this block's feed-forward, or the next block
+            if reader is CAST:
+                return (CAST, ctx.buffer(tag, (T, H), ctx.dtype)) if narrow else None
+            return (reader, ctx.buffer(tag, (T, H), ctx.dtype)) if self._plain_rms(reader) else None
+
+        def leave(then):
+            if then is not None:
+                ctx.leave_normed(after, residual, then[1])
+            elif after is CAST:
+                ctx.leave_normed(CAST, residual, residual)
+
+        h = ctx.take_normed(CAST, residual)
+        if h is None:
+            h = ops.f32_to_bf16(residual, ctx.buffer("stream.cast", (T, H), ctx.dtype)) if narrow else residual
+        last = self.ffn is None
+        then = following(after if last else CAST, "norm.ahead" if last else "norm.inside")
+        add_sublayer(residual, self.mixer.output(h, ctx, site), self.mixer_post, self.mult, following=then)
+        if last:
+            leave(then)
+            return residual
+        h = then[1] if then is not None else residual
+        then = following(after, "norm.ahead")
+        add_sublayer(residual, self.ffn.output(h, ctx), self.ffn_post, self.mult, following=then)
+        leave(then)
+        return residual
+
     def forward(self, residual, ctx, site):
+        if self.reads_stream:
+            return self._forward_stream(residual, ctx, site)
         # the kernel that adds a sublayer's result also makes the norm that reads the residual stream next, where that
         # is an RMS norm over all rows: this block's second norm, or the following block's first (ctx.next_norm), which
         # finds its rows waiting in ctx.normed

@@ -29,7 +29,8 @@ class RotaryEmbedding(Part):
         `scaling` by wavelength (the rule of Llama 3.1): {"factor", "low", "high", "original"}.  A pair whose wavelength
         2 pi / f is shorter than original / high keeps its frequency, one longer than original / low turns `factor`
         times slower, one between goes over linearly in s = (original / wavelength - low) / (high - low):
-        (1 - s) f / factor + s f; cosines and sines keep their size."""
+        (1 - s) f / factor + s f; cosines and sines keep their size.
+        `scaling` linear: {"factor"} alone: every frequency is divided by it (positions shrink), sizes kept."""
         if pairing not in ("split_half", "interleaved"):
             raise ValueError(f"pairing {pairing!r} is neither split_half nor interleaved")
         self.pairing = pairing
@@ -37,8 +38,12 @@ class RotaryEmbedding(Part):
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary size {self.rotary_dim} must be even and at most the head size {head_dim}")
-        self.scaling = self.by_wavelength = None
-        if scaling is not None and ("low" in scaling or "high" in scaling):
+        self.scaling = self.by_wavelength = self.linear = None
+        if scaling is not None and set(scaling) == {"factor"}:
+            self.linear = float(scaling["factor"])
+            if not self.linear > 0:
+                raise ValueError("linear rotary scaling: the factor must be positive")
+        elif scaling is not None and ("low" in scaling or "high" in scaling):
             missing = [k for k in ("factor", "low", "high", "original") if k not in scaling]
             if missing:
                 raise ValueError(f"rotary scaling by wavelength lacks {missing}")
@@ -60,6 +65,8 @@ class RotaryEmbedding(Part):
         half, dims = self.rotary_dim // 2, self.rotary_dim
         index = np.arange(half, dtype=np.float64)
         freq = np.float64(self.theta) ** (-index * 2.0 / dims)
+        if self.linear is not None:
+            return freq / self.linear
         if self.by_wavelength is not None:
             w = self.by_wavelength
             wavelength = 2.0 * math.pi / freq

@@ -318,17 +318,89 @@ class MinGRU(Mixer):
         return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
+class MatrixMemory(Mixer):
+    """The matrix memory of xLSTM (mLSTM): per head a state S [dim, vdim], a normalizer n [dim] and a running maximum m
+    (all zero at a sequence's start), with log gates i = cap tanh((Wi h + bi) / cap) and f = logsigmoid(cap tanh((Wf h +
+    bf) / cap)):  m' = max(f + m, i);  S <- exp(f + m - m') S + exp(i - m') k v^T, n likewise with k alone;
+    o = S^T q / (max(|n . q|, exp(-m')) + 1e-6), q scaled by dim^(-1/2).  Each head's o is divided by its root mean
+    square, times a weight an element, times sigmoid(Wg h), then the output projection.
+
+    n rides in the state as one more column (a value that is always 1), so the recurrence is the linear scan with a
+    decay a head and a step size (ops.linear_scan); the gates, the walk of m and the finish are kernels of their own
+    (ops.mlstm_gates, ops.mlstm_finish).  The state slot holds [heads, dim, vdim + 1] and then m [heads], float."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "i": "i", "f": "f"}
+
+    def __init__(self, name, hidden, heads, dim, vdim, gate_cap, eps, floor=1e-6, names=None):
+        if not gate_cap > 0:
+            raise ValueError("the gates' cap must be positive")
+        self.name, self.hidden, self.heads, self.dim, self.vdim = name, hidden, heads, dim, vdim
+        self.cap, self.eps, self.floor = float(gate_cap), float(eps), float(floor)
+        self.names = {**self.NAMES, **(names or {})}
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return [library.RECURRENCE]
+
+    def state_need(self):
+        return StateNeed((self.heads * self.dim * (self.vdim + 1) + self.heads,), "float32")
+
+    def tensor_specs(self):
+        H, K, V, t = self.hidden, self.heads * self.dim, self.heads * self.vdim, self._tensor
+        return [TensorSpec(t("q"), (K, H)), TensorSpec(t("k"), (K, H)), TensorSpec(t("v"), (V, H)), TensorSpec(t("g"), (V, H)),
+                TensorSpec(t("o"), (H, V)), TensorSpec(t("norm"), (V,), init="one_plus_normal"),
+                TensorSpec(t("i"), (self.heads, H)), TensorSpec(t("i") + ".b", (self.heads,)),
+                TensorSpec(t("f"), (self.heads, H)), TensorSpec(t("f") + ".b", (self.heads,))]
+
+    def bind(self, tensors, dtype):
+        t = self._tensor
+        parts = [matrix_operand(tensors[t(p)], dtype) for p in ("q", "k", "v", "g", "i", "f")]
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_out = matrix_operand(tensors[t("o")], dtype)
+        self.norm_weight = _float(tensors[t("norm")])
+        self.bias_i, self.bias_f = _float(tensors[t("i") + ".b"]), _float(tensors[t("f") + ".b"])
+
+    def output(self, h, ctx, site):
+        T = h.shape[0]
+        nh, R, V = self.heads, self.dim, self.vdim
+        K, W, C = nh * R, nh * V, V + 1
+        proj = ops.gemm(h, self.w_in, ctx.buffer("mm.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        state = ctx.cache.state_storage[site]
+        state = state.view(state.shape[0], -1)
+        decay, step, top = (ctx.buffer("mm." + n, (T, nh), torch.float32) for n in ("decay", "step", "top"))
+        vx = ctx.buffer("mm.vx", (T, nh * C), torch.float32)
+        gates = 2 * K + 2 * W
+        ops.mlstm_gates(proj[:, gates:gates + nh], proj[:, gates + nh:gates + 2 * nh], self.bias_i, self.bias_f, proj[:, 2 * K:2 * K + W],
+                        decay, step, top, vx, state[:, K * C:], ctx.seg_start, ctx.state_slots, nh, V, self.cap)
+        o = ctx.buffer("mm.o", (T, nh * C), torch.float32)
+        _scan(ctx, "mm", proj[:, :K], proj[:, K:2 * K], vx, decay, o, state, nh, R, C, step=step, q_scale=R ** -0.5)
+        act = ops.mlstm_finish(o, top, proj[:, 2 * K + W:2 * K + 2 * W], self.norm_weight, ctx.buffer("mm.act", (T, W), ctx.dtype),
+                               nh, V, self.eps, self.floor)
+        return ops.gemm(act, self.w_out, ctx.buffer("mm.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
+
+
 class SideBySide(Mixer):
     """Two mixers that read the same input; the result is half the sum of theirs, each RMS-normed over the model
-    width with a weight of its own (`<name>.<first_out>` / `<name>.<second_out>`).  At most one of the two keeps pages
-    and at most one a state: a site of the cache has one need of each kind."""
+    width with a weight of its own (`<name>.<first_out>` / `<name>.<second_out>`), or, with `scales` = (a, b), the plain
+    sum a first + b second without norms or tensors of its own.  At most one of the two keeps pages and at most one a
+    state: a site of the cache has one need of each kind."""
 
-    def __init__(self, name, hidden, first, second, eps, first_out="left.out", second_out="right.out"):
+    def __init__(self, name, hidden, first, second, eps, first_out="left.out", second_out="right.out", scales=None):
         for kind in ("cache_need", "state_need"):
             if getattr(first, kind)() is not None and getattr(second, kind)() is not None:
                 raise ValueError(f"both mixers of {name} declare a {kind}: a layer keeps one")
         self.name, self.hidden, self.first, self.second, self.eps = name, hidden, first, second, float(eps)
-        self.out_names = (f"{name}.{first_out}", f"{name}.{second_out}")
+        self.scales = None if scales is None else (float(scales[0]), float(scales[1]))
+        self.out_names = (f"{name}.{first_out}", f"{name}.{second_out}") if scales is None else ()
 
     def mixers(self):
         return [self.first, self.second]
@@ -359,7 +431,9 @@ class SideBySide(Mixer):
             m.prepare(device, dtype)
 
     def output(self, h, ctx, site):
-        from .block import NormedMean
+        from .block import NormedMean, ScaledSum
+        if self.scales is not None:
+            return ScaledSum(self.first.output(h, ctx, site), self.scales[0], self.second.output(h, ctx, site), self.scales[1])
         return NormedMean(self.first.output(h, ctx, site), self.out_weights[0], self.second.output(h, ctx, site),
                           self.out_weights[1], self.eps)
 
@@ -373,3 +447,4 @@ register_part("mixer", "state_space_duality", StateSpaceDuality)
 register_part("mixer", "side_by_side", SideBySide)
 register_part("mixer", "gated_delta_rule", GatedDeltaRule)
 register_part("mixer", "mingru", MinGRU)
+register_part("mixer", "matrix_memory", MatrixMemory)
