@@ -102,10 +102,13 @@ def talking_attention(h, w, p, m, eps):
     return linear(out, w[p + ".o"], w[p + ".o.b"])
 
 
-def matrix_memory(h, w, p, m, eps):
+def matrix_memory(h, w, p, m, eps, margins=None):
     """Matrix memory with exponential gates kept in range by a running maximum (starts at 0), per head:
     m_t = max(f + m, i); S = exp(f + m - m_t) S + exp(i - m_t) k v^T, n likewise with k alone;
-    o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6)."""
+    o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6).
+    `margins`: a list that receives, per token, infinity but for the first: there a head's result is (k . q) v over its
+    own size, that is plus or minus v's direction, and the entry is the smallest |cos(k, q)| over the heads, halved: how
+    far the sign is from turning."""
     T = h.shape[0]
     H, D, V, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
     q = linear(h, w[p + ".q"]).reshape(T, H, D) * D ** -0.5
@@ -123,13 +126,17 @@ def matrix_memory(h, w, p, m, eps):
             n = keep * n + take * k[t, a]
             top = new
             out[t, a] = (q[t, a] @ S) / (max(abs(n @ q[t, a]), math.exp(-top)) + 1e-6)
+    if margins is not None:
+        sign = np.full(T, np.inf)
+        sign[0] = 0.5 * min(abs(q[0, a] @ k[0, a]) / max(np.linalg.norm(q[0, a]) * np.linalg.norm(k[0, a]), 1e-300) for a in range(H))
+        margins.append(sign)
     out = rms(out, eps).reshape(T, H * V) * np.asarray(w[p + ".norm"], np.float64) * sigmoid(linear(h, w[p + ".g"]))
     return linear(out, w[p + ".o"])
 
 
-def parallel_mixer(h, w, p, m, eps):
+def parallel_mixer(h, w, p, m, eps, margins=None):
     return (m["left_scale"] * talking_attention(h, w, p + ".left", m["left"], eps)
-            + m["right_scale"] * matrix_memory(h, w, p + ".right", m["right"], eps))
+            + m["right_scale"] * matrix_memory(h, w, p + ".right", m["right"], eps, margins))
 
 
 # -- feed-forward -------------------------------------------------------------------------------------------------
@@ -144,26 +151,37 @@ def gated_expert(h, w, p):
 
 def route(h, w, p, r, margins=None):
     """Per token the chosen outputs of the router and their weights.  Scores are a softmax over all outputs; the choice
-    adds the correction and is held to the best `keep` of `count` groups of neighbours; the weights are the scores."""
+    adds the correction and is held to the best `keep` of `count` groups of neighbours (a group's score is its largest
+    choice score; the other groups count as minus infinity); the weights are the scores of the chosen, as they are.
+    `margins`: a list that receives, per token, the smallest gap by which a choice was made (between the last group
+    kept and the first one dropped, and between the last output chosen and the first one left out), as a share of the
+    last one taken (about what the two differ by in the router's logits)."""
     z = linear(h, w[p + ".router"])
     e = np.exp(z - z.max(axis=1, keepdims=True))
     s = e / e.sum(axis=1, keepdims=True)
     choice = s + np.asarray(w[p + ".correction"], np.float64)
-    n = choice.shape[1]
+    T, n = choice.shape
+    gap = np.full(T, np.inf)
     groups = r.get("groups")
     if groups is not None:
-        per = n // groups["count"]
-        best = choice.reshape(-1, groups["count"], per).max(axis=2)
-        for t in range(choice.shape[0]):
-            kept = np.argsort(-best[t], kind="stable")[:groups["keep"]]
-            for g in range(groups["count"]):
-                if g not in kept:
-                    choice[t, g * per:(g + 1) * per] = -np.inf
-    picked = np.argsort(-choice, axis=1, kind="stable")[:, :r["top"]]
+        count, keep = groups["count"], groups["keep"]
+        per = n // count
+        best = choice.reshape(T, count, per).max(axis=2)
+        for t in range(T):
+            order = np.argsort(-best[t], kind="stable")
+            if keep < count:
+                gap[t] = (best[t][order[keep - 1]] - best[t][order[keep]]) / max(abs(best[t][order[keep - 1]]), 1e-30)
+            for g in order[keep:]:
+                choice[t, g * per:(g + 1) * per] = -np.inf
+    top = r["top"]
+    picked = np.argsort(-choice, axis=1, kind="stable")[:, :top]
     if margins is not None:
         ordered = -np.sort(-choice, axis=1)
-        finite = np.isfinite(ordered[:, r["top"]]) if n > r["top"] else np.zeros(len(choice), bool)
-        margins.append(np.where(finite, ordered[:, r["top"] - 1] - ordered[:, min(r["top"], n - 1)], np.inf))
+        if n > top:
+            nxt = ordered[:, top]
+            last = np.maximum(np.abs(ordered[:, top - 1]), 1e-30)
+            gap = np.minimum(gap, np.where(np.isfinite(nxt), (ordered[:, top - 1] - np.where(np.isfinite(nxt), nxt, 0.0)) / last, np.inf))
+        margins.append(gap)
     return picked, np.take_along_axis(s, picked, axis=1)
 
 
@@ -184,14 +202,15 @@ def mixture(h, w, p, mlp, margins=None):
 
 def forward(cfg, w, tokens, layers_out=None, margins=None):
     """Logits [T, vocab] of a whole sequence.  `layers_out`: a list that receives the residual stream after every layer;
-    `margins`: a list that receives every router's margins (route)."""
+    `margins`: a list that receives every router's margins (route) and every memory's (matrix_memory): how far a
+    position is from a decision that rounding could turn round."""
     eps = cfg["norm"]["eps"]
     x = np.asarray(w["embed"], np.float64)[np.asarray(tokens)]
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}"
         if layer["type"] != "parallel":
             raise ValueError(f"layer type {layer['type']!r}")
-        x = x + rmsnorm(parallel_mixer(x, w, p + ".mix", layer["mixer"], eps), w[p + ".norm1"], eps)
+        x = x + rmsnorm(parallel_mixer(x, w, p + ".mix", layer["mixer"], eps, margins), w[p + ".norm1"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
             y = dense_ff(x, w, p + ".mlp") if mlp["kind"] == "dense" else mixture(x, w, p + ".mlp", mlp, margins)
