@@ -283,7 +283,7 @@ def main():
     ap.add_argument("--check", type=int, default=1, choices=[0, 1], help="compare the timed way of running with the plain one first")
     ap.add_argument("--widths", default="1024,2048,4096", help="designs workload: model widths to time (comma separated)")
     ap.add_argument("--design-layers", type=int, default=4, help="designs workload: layers of each model")
-    ap.add_argument("--designs", default="llama,novosun,ditazen,noresun", help="designs workload: which designs to time (comma separated)")
+    ap.add_argument("--designs", default="llama,novosun,ditazen,noresun,zovozen", help="designs workload: which designs to time (comma separated)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
@@ -388,7 +388,7 @@ def main():
 
 
 def design_configs(width, layers, context):
-    """A Llama, a Novosun, a Ditazen and a Noresun configuration of the same width, depth and vocabulary.  The Novosun
+    """A Llama, a Novosun, a Ditazen, a Noresun and a Zovozen configuration of the same width, depth and vocabulary.  The Novosun
     layers alternate: softmax attention (heads of 64 for keys, 128 for values, a quarter as many key/value heads) beside
     a state-space layer (inner size twice the width in heads of 64, 128 states, a convolution of 4 taps), then gated
     linear attention (key size half the width, value size the width, in heads of 128 x 256)."""
@@ -428,11 +428,23 @@ def design_configs(width, layers, context):
     noresun = {"architecture": "Noresun", "vocab": vocab, "width": width, "postln_alpha": 2.0, "norm": {"eps": 1e-5},
                "embedding": {"scale": float(width) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 131, "mul_cur": 17}},
                "layers": [order[i % 4] for i in range(layers)], "max_positions": context}
-    return {"llama": llama, "novosun": novosun, "ditazen": ditazen, "noresun": noresun}
+    # Zovozen: attention with scores mixed over the heads (heads of 128, a quarter as many key/value heads, half of a head
+    # turns, blocks of 1,024 positions) beside a matrix memory (as many heads, keys of 64, values of 128) in every layer;
+    # feed-forwards alternate between dense (4 x width, squared relu, biases: 8 width^2) and 14 gated experts of width / 2
+    # plus 2 identity experts in 4 groups of which 2 are kept, 4 chosen, and a shared expert of the width (9 width^2 active)
+    talk = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+            "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 4.0}}}
+    memory = {"heads": heads, "dim": 64, "vdim": 128, "gate_cap": 15.0}
+    pair = {"left": talk, "right": memory, "left_scale": 1.0, "right_scale": 1.0}
+    scored = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 14, "top": 4, "identity": 2, "groups": {"count": 4, "keep": 2}},
+              "shared": {"ff": width}}
+    zovozen = {"architecture": "Zovozen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "max_positions": context,
+               "layers": [{"type": "parallel", "mixer": pair, "mlp": dense if i % 2 == 0 else scored} for i in range(layers)]}
+    return {"llama": llama, "novosun": novosun, "ditazen": ditazen, "noresun": noresun, "zovozen": zovozen}
 
 
 def designs(args):
-    """Prompt steps and decode steps of the Novosun, Ditazen and Noresun designs beside the Llama design at equal width, depth
+    """Prompt steps and decode steps of the Novosun, Ditazen, Noresun and Zovozen designs beside the Llama design at equal width, depth
     and vocabulary (random weights drawn on the device): tokens a second of a whole prompt of --prompt tokens and
     of decode steps of 1, 8 and 64 requests after such prompts, through the step function with captured programs and
     the greedy pick."""
@@ -487,7 +499,7 @@ def designs(args):
             result["prefill"] = {"tokens": prompt, "ms": round(pf * 1e3, 3), "tokens_per_s": round(prompt / pf, 1)}
             out.setdefault(str(width), {})[design] = result
             del runner, model
-    return {"metric": f"prompt and decode tokens/s of the Novosun, Ditazen and Noresun designs beside Llama at equal width, {args.design_layers} layers",
+    return {"metric": f"prompt and decode tokens/s of the Novosun, Ditazen, Noresun and Zovozen designs beside Llama at equal width, {args.design_layers} layers",
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "steps": steps,
             "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "prompt_len": prompt,
             "execution": args.execution, "widths": out}

@@ -10,8 +10,9 @@
 // its results.
 //
 //   gates      i_t = cap tanh((zi + bi) / cap), f_t = logsigmoid(cap tanh((zf + bf) / cap)) from the projections' float
-//              results; the walk of m along a segment's rows (a thread a head; the maximum is the only chain); decay,
-//              step and m_t a row and head; the values with their column of ones; m kept in the state slot
+//              results and the values with their column of ones (a block a row); then the walk of m along a segment's
+//              rows (a wave a segment and head, the rows dealt to its lanes in runs): decay, step and m_t a row and
+//              head; m kept in the state slot
 //   finish     o / denominator, each head divided by its root mean square, times a weight an element, times
 //              sigmoid(gate), into the activations' type
 // Everything here is float arithmetic.
@@ -19,52 +20,74 @@
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-// One block a segment.  zi / zf: [T, heads] views (row strides ldi / ldf); v [T, heads * V] (ldv); decay, step, top
-// [T, heads]; vx [T, heads * (V + 1)]; m of a request at state + slot * slot_stride + head.
+// One block a row: the log gates of the row's heads (i into `step`, f into `decay`, for the walk below to turn into
+// factors) and the row's values with their column of ones.  zi / zf: [T, heads] views (row strides ldi / ldf);
+// v [T, heads * V] (ldv); vx [T, heads * (V + 1)].
 __global__ void __launch_bounds__(256)
-mlstm_gates_kernel(const float* __restrict__ zi, int ldi, const float* __restrict__ zf, int ldf, const float* __restrict__ bi,
-                   const float* __restrict__ bf, const float* __restrict__ v, int ldv, float* __restrict__ decay,
-                   float* __restrict__ step, float* __restrict__ top, float* __restrict__ vx, float* __restrict__ state,
-                   long long slot_stride, const int* __restrict__ seg_start, const int* __restrict__ state_slots, int heads, int V,
-                   float cap) {
-    const int seg = blockIdx.x;
-    const int s0 = seg_start[seg], s1 = seg_start[seg + 1];
-    if (s1 <= s0) return;                                            // (padding of a captured step)
-    const int n = s1 - s0, C = V + 1;
-    for (int i = threadIdx.x; i < n * heads; i += 256) {
-        const int t = s0 + i / heads, h = i % heads;
-        step[(size_t)t * heads + h] = cap * tanhf((zi[(size_t)t * ldi + h] + bi[h]) / cap);
-        decay[(size_t)t * heads + h] = log_sigmoid(cap * tanhf((zf[(size_t)t * ldf + h] + bf[h]) / cap));
+mlstm_rows_kernel(const float* __restrict__ zi, int ldi, const float* __restrict__ zf, int ldf, const float* __restrict__ bi,
+                  const float* __restrict__ bf, const float* __restrict__ v, int ldv, float* __restrict__ decay,
+                  float* __restrict__ step, float* __restrict__ vx, int heads, int V, float cap) {
+    const size_t t = blockIdx.x;
+    const int C = V + 1;
+    for (int h = threadIdx.x; h < heads; h += 256) {
+        step[t * heads + h] = cap * tanhf((zi[t * ldi + h] + bi[h]) / cap);
+        decay[t * heads + h] = log_sigmoid(cap * tanhf((zf[t * ldf + h] + bf[h]) / cap));
     }
-    for (size_t i = threadIdx.x; i < (size_t)n * heads * C; i += 256) {
-        const size_t t = s0 + i / ((size_t)heads * C);
-        const int hc = (int)(i % ((size_t)heads * C)), h = hc / C, c = hc % C;
+    for (int hc = threadIdx.x; hc < heads * C; hc += 256) {
+        const int h = hc / C, c = hc % C;
         vx[t * heads * C + hc] = c < V ? v[t * ldv + h * V + c] : 1.0f;
     }
-    __syncthreads();
-    float* ms = state + (long long)state_slots[seg] * slot_stride;
-    for (int h = threadIdx.x; h < heads; h += 256) {
-        float m = ms[h];
-        for (int t = s0; t < s1; ++t) {
-            const float f = decay[(size_t)t * heads + h], i = step[(size_t)t * heads + h];
-            const float m_new = fmaxf(f + m, i);
-            decay[(size_t)t * heads + h] = expf(f + m - m_new);
-            step[(size_t)t * heads + h] = expf(i - m_new);
-            top[(size_t)t * heads + h] = m_new;
-            m = m_new;
-        }
-        ms[h] = m;
+}
+
+// The walk of the running maximum, a wave a (segment, head): m' = max(f + m, i) along the segment's rows is the map
+// x -> max(a + x, b) with (a, b) = (f, i), and two such maps compose to one: later o earlier = (a1 + a2, max(a2 + b1,
+// b2)).  A lane composes its run of consecutive rows, the lanes' maps meet in a scan over the wave, and every lane walks
+// its run again from the maximum it starts with, turning the log gates into the factors of the state's update
+// (decay = exp(f + m - m'), step = exp(i - m')) and leaving m' (`top`).  m of a request at state + slot * slot_stride + head.
+__global__ void __launch_bounds__(64)
+mlstm_walk_kernel(float* __restrict__ decay, float* __restrict__ step, float* __restrict__ top, float* __restrict__ state,
+                  long long slot_stride, const int* __restrict__ seg_start, const int* __restrict__ state_slots, int heads) {
+    const int seg = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int s0 = seg_start[seg], s1 = seg_start[seg + 1];
+    if (s1 <= s0) return;                                            // (padding of a captured step)
+    float* ms = state + (long long)state_slots[seg] * slot_stride + h;
+    const int n = s1 - s0, per = (n + WAVE - 1) / WAVE;
+    const int t0 = min(s0 + lane * per, s1), t1 = min(t0 + per, s1);
+    float A = 0.f, B = -INFINITY;                                    // the identity map
+    for (int t = t0; t < t1; ++t) {
+        const float f = decay[(size_t)t * heads + h], i = step[(size_t)t * heads + h];
+        B = fmaxf(f + B, i);
+        A += f;
     }
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) {
+        const float Ap = __shfl_up(A, off, WAVE), Bp = __shfl_up(B, off, WAVE);
+        if (lane >= off) { B = fmaxf(A + Bp, B); A += Ap; }
+    }
+    const float m0 = *ms;
+    const float Ab = __shfl_up(A, 1, WAVE), Bb = __shfl_up(B, 1, WAVE);
+    float m = lane == 0 ? m0 : fmaxf(Ab + m0, Bb);                   // the maximum before this lane's first row
+    for (int t = t0; t < t1; ++t) {
+        const float f = decay[(size_t)t * heads + h], i = step[(size_t)t * heads + h];
+        const float m_new = fmaxf(f + m, i);
+        decay[(size_t)t * heads + h] = expf(f + m - m_new);
+        step[(size_t)t * heads + h] = expf(i - m_new);
+        top[(size_t)t * heads + h] = m_new;
+        m = m_new;
+    }
+    if (t1 == s1 && t0 < t1) *ms = m;                                // (the lane of the segment's last row)
 }
 
 extern "C" int cisr_mlstm_gates(const float* zi, int ldi, const float* zf, int ldf, const float* bi, const float* bf, const float* v,
                                 int ldv, float* decay, float* step, float* top, float* vx, float* state, long long slot_stride,
-                                const int* seg_start, const int* state_slots, int segments, int heads, int V, float cap,
+                                const int* seg_start, const int* state_slots, int rows, int segments, int heads, int V, float cap,
                                 hipStream_t stream) {
-    if (segments <= 0) return 0;
-    if (heads <= 0 || V <= 0 || !(cap > 0.f)) return (int)hipErrorInvalidValue;
-    mlstm_gates_kernel<<<segments, 256, 0, stream>>>(zi, ldi, zf, ldf, bi, bf, v, ldv, decay, step, top, vx, state, slot_stride,
-                                                     seg_start, state_slots, heads, V, cap);
+    if (segments <= 0 || rows <= 0) return 0;
+    if (heads <= 0 || heads > 65535 || V <= 0 || !(cap > 0.f)) return (int)hipErrorInvalidValue;
+    mlstm_rows_kernel<<<rows, 256, 0, stream>>>(zi, ldi, zf, ldf, bi, bf, v, ldv, decay, step, vx, heads, V, cap);
+    int err = CISR_LAUNCH_CHECK();
+    if (err) return err;
+    mlstm_walk_kernel<<<dim3(segments, heads), 64, 0, stream>>>(decay, step, top, state, slot_stride, seg_start, state_slots, heads);
     return CISR_LAUNCH_CHECK();
 }
 

@@ -371,13 +371,43 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
     return None
 
 
+def talking_units(dtype, heads, kv_heads, vdim, pad):
+    """Names of the shared objects that the attention with mixed scores needs beside the core."""
+    from . import library
+    return [library.TALKING] if ops.talking_tiles_ok(dtype, heads, kv_heads, vdim, pad, 8) else []
+
+
+def talking_splits(tiles, span):
+    """Blocks that share a tile's keys in the tile form of the attention with mixed scores.  A tile is one block of at
+    most eight waves with three barriers a 32-key step, so a compute unit wants two or three blocks to have something to
+    run while one waits: the keys are split until the launch has a block for every compute unit, each keeping at least
+    four steps.  (2,048 rows of 16 heads of 128 over blocks of 1,024 positions, 129 tiles: 326 us unsplit, 190 with two
+    blocks a tile, 193 to 203 with three to six, 227 with eight: the sums that the merge reads grow with the split.)"""
+    steps = max(1, -(-span // 32))
+    return int(max(1, min(-(-256 // max(tiles, 1)), steps // 4, 8)))
+
+
 def talking_attention(ctx, q, kcache, vcache, view, out, heads, kv_heads, vdim, pad, mix, scale, temp=None, sink=None,
                       window=None, chunk=None, gate=None):
     """out[r] = attention of row r over its request's cached keys where the scores of all heads of a row are mixed
     (`mix` [heads, heads], after `temp`[g] scale) before the softmax, whose denominator holds exp(`sink`[h]) as well; a
     row sees its block of `chunk` positions up to itself (or the last `window` keys, or all); `gate`: the result times
-    sigmoid(gate) element by element.  The mix needs every head's score of a (row, key) pair in one place, so this is a
-    kernel of its own beside the paged attention above: one block a row walks the row's keys for all heads."""
+    sigmoid(gate) element by element.  The mix needs every head's score of a (row, key) pair in one place, so these are
+    kernels of their own beside the paged attention above: steps with prompt portions in bfloat16 run tiles of 16 rows
+    with all their heads on the matrix cores (the task list of the paged attention's tiles serves); steps of single
+    tokens, float32 and sizes the tiles do not take run the exact kernel, one block a row."""
+    if not ctx.decode_only and ops.talking_tiles_ok(out.dtype, heads, kv_heads, vdim, pad, view.page_size):
+        tasks, _ = ctx.step_array(TileTasks(ops.TALKING_TILE_ROWS))
+        rows = out.shape[0]
+        splits = talking_splits(tasks.numel() // 4, min(ctx.span_hint, chunk or window or ctx.span_hint))
+        workspace = None
+        if splits > 1:
+            workspace = (ctx.buffer("tattn.part_o", (rows * heads * splits * vdim,), torch.float32),
+                         ctx.buffer("tattn.part_ml", (rows * heads * splits * 2,), torch.float32))
+        ops.attention_talking_tiles(q, kcache, vcache, view.tables, tasks.view(-1, 4), ctx.positions, out, heads, kv_heads, vdim, pad,
+                                    view.page_size, mix, scale, temp=temp, sink=sink, window=window, chunk=chunk, gate=gate,
+                                    splits=splits, workspace=workspace)
+        return out
     ops.attention_talking(q, q.stride(0), kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out, heads, kv_heads, vdim, pad,
                           view.page_size, mix, scale, temp=temp, sink=sink, window=window, chunk=chunk, gate=gate)
     return out

@@ -39,6 +39,7 @@ MEASURE = "measure"                                # kernels that only measure t
 RECURRENCE = "recurrence"                          # mixers with a state per request: scans, short convolutions, their gates
 OWN_UNITS = (MEASURE, RECURRENCE)                  # units of the source files whose names start with the unit's
 ATTENTION_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
+TALKING = "attn_talk"                              # the matrix-core attention whose scores are mixed over the heads (attention_mfma_talk.hip)
 
 
 class KernelLibraryError(RuntimeError):
@@ -58,7 +59,7 @@ def attention_unit(dpad, law="softmax"):
 def units():
     """The shared objects the kernels are built into: the core, and one per padded head size of the
     matrix-core attention (a model needs only its own, so a first call compiles only that one)."""
-    return [CORE, *OWN_UNITS] + [attention_unit(d, law) for law in ("softmax", "sigmoid") for d in ATTENTION_PADS]
+    return [CORE, *OWN_UNITS, TALKING] + [attention_unit(d, law) for law in ("softmax", "sigmoid") for d in ATTENTION_PADS]
 
 
 def sources(unit=CORE):

@@ -401,6 +401,66 @@ def attention_talking(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
     return out
 
 
+_talking = None
+
+
+def _talk():
+    global _talking
+    if _talking is None:
+        h = library.load(library.TALKING)
+        p, i, f = C.c_void_p, C.c_int, C.c_float
+        h.cisr_attn_talking_tiles.argtypes = [p, i, p, p, p, p, i, p, p, p, p, p, i, p, i, i, i, i, i, i, i, i, f, i, i, p, p, p]
+        h.cisr_attn_talking_tiles.restype = C.c_int
+        _talking = h
+    return _talking
+
+
+TALKING_TILE_ROWS = 16     # rows of a tile of attention_talking_tiles
+
+
+def talking_tiles_ok(dtype, heads, kv_heads, vdim, pad, page_size):
+    """Whether attention_talking_tiles takes these sizes: bfloat16, at most 32 heads of at most 128 coordinates, pages
+    of a multiple of 8 keys."""
+    return (dtype == torch.bfloat16 and 0 < heads <= 32 and kv_heads > 0 and heads % kv_heads == 0 and 0 < pad <= 128 and pad % 8 == 0
+            and 0 < vdim <= pad and page_size > 0 and page_size % 8 == 0)
+
+
+def attention_talking_tiles(q, kcache, vcache, tables, tasks, positions, out, heads, kv_heads, vdim, pad, page_size, mix, scale,
+                            temp=None, sink=None, window=None, chunk=None, gate=None, splits=1, workspace=None):
+    """attention_talking on the matrix cores for bfloat16: `tasks` int32 [n, 4] lists tiles of up to 16 consecutive rows of
+    one segment (segment, first row, rows, anything; segment -1: no tile); a block takes a tile with all its heads.
+    `splits` > 1: that many blocks share a tile's keys and leave their sums in `workspace` = (float [T * heads * splits *
+    vdim], float [T * heads * splits * 2]) for a merge kernel that runs behind them."""
+    rows = out.shape[0]
+    pages = kcache.shape[0]
+    if not talking_tiles_ok(out.dtype, heads, kv_heads, vdim, pad, page_size):
+        raise KernelError("attention_talking_tiles: sizes not supported")
+    gp, ldg = None, 0
+    if gate is not None:
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (rows, heads * vdim) or gate.stride(1) != 1 or not gate.is_cuda:
+            raise KernelError("attention_talking_tiles: the gate must be float [T, heads * vdim] with unit stride")
+        gp, ldg = gate.data_ptr(), gate.stride(0)
+    if q.dim() != 2 or q.shape[0] != rows or q.stride(1) != 1 or q.shape[1] < heads * pad or q.dtype != out.dtype or not q.is_cuda or q.stride(0) % 8:
+        raise KernelError("attention_talking_tiles: q must be bf16 [T, >= heads * pad] with rows of 16-byte chunks")
+    if tasks.dtype != torch.int32 or tasks.dim() != 2 or tasks.shape[1] != 4 or not tasks.is_contiguous() or not tasks.is_cuda:
+        raise KernelError("attention_talking_tiles: tasks must be int32 [n, 4]")
+    po = pm = None
+    if splits > 1:
+        if workspace is None or workspace[0].numel() < rows * heads * splits * vdim or workspace[1].numel() < rows * heads * splits * 2:
+            raise KernelError("attention_talking_tiles: split keys need a workspace for their sums")
+        po, pm = _dev(workspace[0], "part_o", torch.float32), _dev(workspace[1], "part_ml", torch.float32)
+    _check(_talk().cisr_attn_talking_tiles(q.data_ptr(), q.stride(0), _dev(kcache, "kcache", out.dtype, (pages, kv_heads, page_size, pad)),
+                                           _dev(vcache, "vcache", out.dtype, (pages, kv_heads, pad, page_size)), _dev(tables, "tables", torch.int32),
+                                           tasks.data_ptr(), tasks.shape[0], _dev(positions, "positions", torch.int32, (rows,)),
+                                           _dev(mix, "mix", torch.float32, (heads, heads)),
+                                           None if temp is None else _dev(temp, "temp", torch.float32, (heads,)),
+                                           None if sink is None else _dev(sink, "sink", torch.float32, (heads,)), gp, ldg,
+                                           _dev(out, "out", torch.bfloat16, (rows, heads * vdim)), heads, kv_heads, vdim, pad, page_size,
+                                           tables.shape[1], int(window or 0), int(chunk or 0), float(scale), rows, int(splits), po, pm,
+                                           _stream()), "attention_talking_tiles")
+    return out
+
+
 class ScratchPool:
     """Device memory that some products need beyond their inputs and outputs: the library's bf16 product before its
     sum into the residual, the wide kernel's partial sums, the slice winners of the argmax.  A buffer is handed out
@@ -1184,7 +1244,7 @@ def _rec():
             "cisr_delta_scan": [p, i, p, i, p, i, p, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
             "cisr_unit_heads": [p, i, i, i, i, i, f, f, p],
             "cisr_mingru_scan": [p, i, p, p, p, i, p, p, p, i, i, i, i, p, i, i, p],
-            "cisr_mlstm_gates": [p, i, p, i, p, p, p, i, p, p, p, p, p, ll, p, p, i, i, i, f, p],
+            "cisr_mlstm_gates": [p, i, p, i, p, p, p, i, p, p, p, p, p, ll, p, p, i, i, i, i, f, p],
             "cisr_mlstm_finish": [p, p, p, i, p, p, i, i, i, f, f, i, p],
         }
         for name, args in sig.items():
@@ -1636,7 +1696,7 @@ def mlstm_gates(zi, zf, bias_i, bias_f, v, decay, step, top, vx, top_state, seg_
                                    vp, ldv, _dev(decay, "decay", torch.float32, (T, heads)), _dev(step, "step", torch.float32, (T, heads)),
                                    _dev(top, "top", torch.float32, (T, heads)), _dev(vx, "vx", torch.float32, (T, heads * (vdim + 1))),
                                    top_state.data_ptr(), top_state.stride(0), _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
-                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, vdim, float(cap), _stream()),
+                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), T, segments, heads, vdim, float(cap), _stream()),
            "mlstm_gates")
 
 

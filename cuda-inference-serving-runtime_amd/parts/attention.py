@@ -472,6 +472,12 @@ class TalkingAttention(Mixer):
     def _tensor(self, which):
         return f"{self.name}.{self.names[which]}"
 
+    def kernel_units(self, dtype):
+        return kernel.talking_units(dtype, self.heads, self.kv_heads, self.vdim, self.pad)
+
+    def step_arrays(self):
+        return [kernel.TileTasks(ops.TALKING_TILE_ROWS)]
+
     def cache_need(self):
         return KVNeed(self.kv_heads, self.pad) if self.chunk is None else ChunkNeed(self.kv_heads, self.pad, self.chunk, self.chunk)
 
