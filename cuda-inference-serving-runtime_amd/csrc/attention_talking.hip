@@ -15,7 +15,8 @@
 // Keys are walked 64 at a time, tiles at absolute multiples of 64: (1) a thread a (key head, key) makes the raw scores
 // of the head's group, 16 bytes of the key row a load; (2) a thread a (head, key) mixes; (3) a wave a head moves the
 // running maximum and denominator; (4) a thread an output coordinate (E of them in registers) adds the tile's values,
-// eight keys of a transposed value page a load where pages hold a multiple of eight keys.
+// eight keys of a transposed value page a load where pages hold a multiple of eight keys.  With `splits` > 1 that
+// many blocks share a row's tiles (steps of few rows: one block a row leaves the GPU empty) and a small kernel merges.
 #include "common.h"
 
 #define TK_KEYS 64
@@ -29,6 +30,7 @@ struct TalkArgs {
     void* out;
     int heads, kv_heads, vdim, pad, page_size, width, window, chunk;
     float scale;
+    int splits; float* part_o; float* part_ml;      // splits > 1: block (row, s) walks the tiles s, s + splits, ... and leaves sums
 };
 
 __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
@@ -70,7 +72,15 @@ attn_talking_kernel(TalkArgs p) {
         end = pos + 1;
         begin = p.chunk > 0 ? (pos / p.chunk) * p.chunk : (p.window > 0 && end > p.window) ? end - p.window : 0;
     }
+    const int split = blockIdx.y, S = p.splits;
     if (begin >= end) {
+        if (S > 1) {                                  // (nothing to merge: every block along the keys says so)
+            for (int h = tid; h < H; h += 256) {
+                const size_t part = ((size_t)row * H + h) * S + split;
+                p.part_ml[part * 2] = -INFINITY; p.part_ml[part * 2 + 1] = 0.f;
+            }
+            return;
+        }
 #pragma unroll
         for (int e = 0; e < E; ++e) { const int i = tid + 256 * e; if (i < n_out) store_f32(out + i, 0.f); }
         return;
@@ -79,14 +89,15 @@ attn_talking_kernel(TalkArgs p) {
     for (int i = tid; i < H * pad; i += 256) qs[i] = load_f32(qr + i);
     for (int i = tid; i < H * H; i += 256) mixw[i] = p.mix[i] * (p.temp ? p.temp[i % H] : 1.0f) * p.scale;
     for (int h = tid; h < H; h += 256) {
-        run_m[h] = p.sink ? p.sink[h] : -INFINITY;        // the sink: a key of score sink_h and no value
-        run_l[h] = p.sink ? 1.0f : 0.f;
+        const bool sunk = p.sink && split == 0;           // the sink: a key of score sink_h and no value; it counts once
+        run_m[h] = sunk ? p.sink[h] : -INFINITY;
+        run_l[h] = sunk ? 1.0f : 0.f;
     }
     const int* table = p.tables + (size_t)seg * p.width;
     const T* kc = (const T*)p.kcache;
     const T* vc = (const T*)p.vcache;
     const bool by8 = P % 8 == 0;
-    for (int base = begin / TK_KEYS * TK_KEYS; base < end; base += TK_KEYS) {
+    for (int base = begin / TK_KEYS * TK_KEYS + split * TK_KEYS; base < end; base += S * TK_KEYS) {
         __syncthreads();                      // (the tile before is done with pg, po, pw, alpha; the first: qs, mixw are there)
         if (tid < TK_KEYS) {
             const int t = base + tid;
@@ -170,6 +181,20 @@ attn_talking_kernel(TalkArgs p) {
         }
     }
     __syncthreads();
+    if (S > 1) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int i = tid + 256 * e;
+            if (i >= n_out) continue;
+            const int h = i / p.vdim, d = i % p.vdim;
+            p.part_o[(((size_t)row * H + h) * S + split) * p.vdim + d] = acc[e];
+        }
+        for (int h = tid; h < H; h += 256) {
+            const size_t part = ((size_t)row * H + h) * S + split;
+            p.part_ml[part * 2] = run_m[h]; p.part_ml[part * 2 + 1] = run_l[h];
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int i = tid + 256 * e;
@@ -181,6 +206,32 @@ attn_talking_kernel(TalkArgs p) {
     }
 }
 
+// The blocks along a row's keys leave o_s = sum_j exp(s_j - m_s) v_j, m_s and l_s; with m = max m_s the row's result is
+// sum_s exp(m_s - m) o_s / sum_s exp(m_s - m) l_s, times sigmoid(gate).  A block a (row, head).
+template <typename T>
+__global__ void __launch_bounds__(128)
+talking_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, const float* __restrict__ gate, int ldg,
+                     T* __restrict__ out, int heads, int vdim, int splits) {
+    const size_t row = blockIdx.x;
+    const int h = blockIdx.y;
+    const size_t base = (row * heads + h) * splits;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
+    for (int c = threadIdx.x; c < vdim; c += 128) {
+        float num = 0.f, den = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float ms = part_ml[(base + s) * 2];
+            if (ms == -INFINITY) continue;                       // (a block that saw no key of this row)
+            const float w = expf(ms - m);
+            num += w * part_o[(base + s) * vdim + c];
+            den += w * part_ml[(base + s) * 2 + 1];
+        }
+        float v = den > 0.f ? num / den : 0.f;
+        if (gate) v *= 1.0f / (1.0f + expf(-gate[row * ldg + h * vdim + c]));
+        store_f32(out + row * heads * vdim + h * vdim + c, v);
+    }
+}
+
 static size_t talking_lds(int heads, int pad) {
     return ((size_t)heads * pad + (size_t)heads * heads + 2 * (size_t)heads * TK_KEYS + 3 * (size_t)heads) * sizeof(float) + 2 * TK_KEYS * sizeof(int);
 }
@@ -189,7 +240,8 @@ template <typename T>
 static int launch_talking(const TalkArgs& a, int rows, hipStream_t stream) {
     const size_t lds = talking_lds(a.heads, a.pad);
     const int per = (a.heads * a.vdim + 255) / 256;
-#define TALK(E) attn_talking_kernel<T, E><<<rows, 256, lds, stream>>>(a)
+    const dim3 grid(rows, a.splits);
+#define TALK(E) attn_talking_kernel<T, E><<<grid, 256, lds, stream>>>(a)
     if (per <= 2) TALK(2);
     else if (per <= 4) TALK(4);
     else if (per <= 8) TALK(8);
@@ -197,18 +249,23 @@ static int launch_talking(const TalkArgs& a, int rows, hipStream_t stream) {
     else if (per <= 32) TALK(32);
     else return (int)hipErrorInvalidValue;
 #undef TALK
+    const int err = CISR_LAUNCH_CHECK();
+    if (err || a.splits == 1) return err;
+    talking_merge_kernel<T><<<dim3(rows, a.heads), 128, 0, stream>>>(a.part_o, a.part_ml, a.gate, a.ldg, (T*)a.out, a.heads, a.vdim, a.splits);
     return CISR_LAUNCH_CHECK();
 }
 
 extern "C" int cisr_attn_talking(const void* q, int q_row_stride, const void* kcache, const void* vcache, const int* tables,
                                  const int* seg_of_row, const int* positions, const float* mix, const float* temp, const float* sink,
                                  const float* gate, int ldg, void* out, int rows, int heads, int kv_heads, int vdim, int pad,
-                                 int page_size, int width, int window, int chunk, float scale, int dtype, hipStream_t stream) {
+                                 int page_size, int width, int window, int chunk, float scale, int splits, float* part_o, float* part_ml,
+                                 int dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
+    if (splits < 1 || splits > 65535 || heads > 65535 || (splits > 1 && (!part_o || !part_ml))) return (int)hipErrorInvalidValue;
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || pad <= 0 || pad % 8 || vdim <= 0 || vdim > pad || page_size <= 0 ||
         !mix || talking_lds(heads, pad) > 64 * 1024 || q_row_stride < heads * pad || (gate && ldg < heads * vdim))
         return (int)hipErrorInvalidValue;
     const TalkArgs a = {q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, mix, temp, sink, gate, ldg, out,
-                        heads, kv_heads, vdim, pad, page_size, width, window, chunk, scale};
+                        heads, kv_heads, vdim, pad, page_size, width, window, chunk, scale, splits, part_o, part_ml};
     return dtype == DT_F32 ? launch_talking<float>(a, rows, stream) : launch_talking<bf16_t>(a, rows, stream);
 }

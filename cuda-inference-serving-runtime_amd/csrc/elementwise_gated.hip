@@ -19,15 +19,16 @@ __global__ void __launch_bounds__(256)
 post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
                      const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
                      int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out,
-                     float ca, float cb) {
+                     float ca, float cb, const float* __restrict__ bias_a) {
     __shared__ float red[4];
     extern __shared__ float kept[];
     const size_t row = blockIdx.x;
     const float* ar = a + row * dim;
     const float* br = TWO ? b + row * dim : nullptr;
+    auto first = [&](int d) { return bias_a ? ar[d] + bias_a[d] : ar[d]; };     // (a bias a column that the product left out)
     float sa = 0.f, sb = 0.f;
     for (int d = threadIdx.x; d < dim; d += 256) {
-        const float u = ar[d];
+        const float u = first(d);
         sa += u * u;
         if (TWO) { const float v = br[d]; sb += v * v; }
         else if (KEEP) kept[d] = u;
@@ -38,7 +39,7 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
         rb = wa ? 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps) : cb;
         sa = 0.f;
         for (int d = threadIdx.x; d < dim; d += 256) {
-            const float y = ar[d] * ra * (wa ? wa[d] : 1.0f) + br[d] * rb * (wa ? wb[d] : 1.0f);
+            const float y = first(d) * ra * (wa ? wa[d] : 1.0f) + br[d] * rb * (wa ? wb[d] : 1.0f);
             if (KEEP) kept[d] = y;
             sa += y * y;
         }
@@ -48,7 +49,7 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
     float* xr = x + row * dim;
     float sn = 0.f;
     for (int d = threadIdx.x; d < dim; d += 256) {         // (a thread reads back only what it wrote itself)
-        const float y = KEEP ? kept[d] : TWO ? ar[d] * ra * (wa ? wa[d] : 1.0f) + br[d] * rb * (wa ? wb[d] : 1.0f) : ar[d];
+        const float y = KEEP ? kept[d] : TWO ? first(d) * ra * (wa ? wa[d] : 1.0f) + br[d] * rb * (wa ? wb[d] : 1.0f) : first(d);
         const float xn = xr[d] + y * scale * (w ? w[d] : 1.0f);
         xr[d] = xn;
         if (KEEP) kept[d] = xn;
@@ -68,7 +69,7 @@ __global__ void __launch_bounds__(256)
 post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
                            const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
                            int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out,
-                           int slices_a, int slices_b, float ca, float cb) {
+                           int slices_a, int slices_b, float ca, float cb, const float* __restrict__ bias_a) {
     __shared__ float red[4];
     const size_t row = blockIdx.x;
     float va[E], vb[E], vx[E], vw[E], vwa[E], vwb[E], vn[E];
@@ -102,6 +103,10 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
     };
     if (slices_a > 1) add_slices(va, a, slices_a);
     if (TWO && slices_b > 1) add_slices(vb, b, slices_b);
+    if (bias_a) {                                             // (a bias a column that the product left out)
+#pragma unroll
+        for (int e = 0; e < E; ++e) { const int d = threadIdx.x + 256 * e; if (d < dim) va[e] += bias_a[d]; }
+    }
     float sa = 0.f, sb = 0.f;
 #pragma unroll
     for (int e = 0; e < E; ++e) { sa += va[e] * va[e]; if (TWO) sb += vb[e] * vb[e]; }
@@ -132,29 +137,30 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
 template <bool TWO, typename T>
 static void launch_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb, const float* w,
                                  int rows, int dim, float eps, float mult, const float* next_w, float next_eps, T* next_out,
-                                 int slices_a, int slices_b, float ca, float cb, hipStream_t stream) {
-#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, slices_a, slices_b, ca, cb)
+                                 int slices_a, int slices_b, float ca, float cb, const float* bias_a, hipStream_t stream) {
+#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, slices_a, slices_b, ca, cb, bias_a)
     if (dim <= 1024) SHORT(4);
     else if (dim <= 2048) SHORT(8);
     else if (dim <= 4096) SHORT(16);
 #undef SHORT
-    else if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, ca, cb);
-    else post_norm_add_kernel<TWO, false, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, ca, cb);
+    else if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, ca, cb, bias_a);
+    else post_norm_add_kernel<TWO, false, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, ca, cb, bias_a);
 }
 
 extern "C" int cisr_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb,
                                   const float* w, int rows, int dim, float eps, float mult, const float* next_w, float next_eps,
-                                  void* next_out, int next_dtype, int slices_a, int slices_b, float ca, float cb, hipStream_t stream) {
+                                  void* next_out, int next_dtype, int slices_a, int slices_b, float ca, float cb, const float* bias_a,
+                                  hipStream_t stream) {
     if (rows <= 0) return 0;
     if (dim <= 0 || (b != nullptr && ((wa == nullptr) != (wb == nullptr))) || (next_w != nullptr && next_out == nullptr) ||
         slices_a < 0 || slices_b < 0 || ((slices_a > 0 || slices_b > 0) && dim > 4096))    // (partial sums: the kernel of short rows)
         return (int)hipErrorInvalidValue;
     if (next_dtype == DT_F32) {
-        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, ca, cb, stream);
-        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, ca, cb, stream);
+        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, ca, cb, bias_a, stream);
+        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, ca, cb, bias_a, stream);
     } else {
-        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, ca, cb, stream);
-        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, ca, cb, stream);
+        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, ca, cb, bias_a, stream);
+        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, ca, cb, bias_a, stream);
     }
     return CISR_LAUNCH_CHECK();
 }

@@ -23,15 +23,29 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 // One block a row: the log gates of the row's heads (i into `step`, f into `decay`, for the walk below to turn into
 // factors) and the row's values with their column of ones.  zi / zf: [T, heads] views (row strides ldi / ldf);
 // v [T, heads * V] (ldv); vx [T, heads * (V + 1)].
+// SINGLE: every segment has one row (row t is segment t), and the thread that makes a head's gates moves the head's
+// running maximum on as well: no walk behind this kernel.
+template <bool SINGLE>
 __global__ void __launch_bounds__(256)
 mlstm_rows_kernel(const float* __restrict__ zi, int ldi, const float* __restrict__ zf, int ldf, const float* __restrict__ bi,
                   const float* __restrict__ bf, const float* __restrict__ v, int ldv, float* __restrict__ decay,
-                  float* __restrict__ step, float* __restrict__ vx, int heads, int V, float cap) {
+                  float* __restrict__ step, float* __restrict__ vx, int heads, int V, float cap, float* __restrict__ top,
+                  float* __restrict__ state, long long slot_stride, const int* __restrict__ seg_start,
+                  const int* __restrict__ state_slots, int segments) {
     const size_t t = blockIdx.x;
     const int C = V + 1;
+    const bool live = SINGLE && (int)t < segments && seg_start[t + 1] > seg_start[t];        // (else: padding of a captured step)
     for (int h = threadIdx.x; h < heads; h += 256) {
-        step[t * heads + h] = cap * tanhf((zi[t * ldi + h] + bi[h]) / cap);
-        decay[t * heads + h] = log_sigmoid(cap * tanhf((zf[t * ldf + h] + bf[h]) / cap));
+        const float i = cap * tanhf((zi[t * ldi + h] + bi[h]) / cap);
+        const float f = log_sigmoid(cap * tanhf((zf[t * ldf + h] + bf[h]) / cap));
+        if (!SINGLE) { step[t * heads + h] = i; decay[t * heads + h] = f; continue; }
+        if (!live) continue;
+        float* ms = state + (long long)state_slots[t] * slot_stride + h;
+        const float m = *ms, m_new = fmaxf(f + m, i);
+        decay[t * heads + h] = expf(f + m - m_new);
+        step[t * heads + h] = expf(i - m_new);
+        top[t * heads + h] = m_new;
+        *ms = m_new;
     }
     for (int hc = threadIdx.x; hc < heads * C; hc += 256) {
         const int h = hc / C, c = hc % C;
@@ -81,10 +95,16 @@ mlstm_walk_kernel(float* __restrict__ decay, float* __restrict__ step, float* __
 extern "C" int cisr_mlstm_gates(const float* zi, int ldi, const float* zf, int ldf, const float* bi, const float* bf, const float* v,
                                 int ldv, float* decay, float* step, float* top, float* vx, float* state, long long slot_stride,
                                 const int* seg_start, const int* state_slots, int rows, int segments, int heads, int V, float cap,
-                                hipStream_t stream) {
+                                int single_rows, hipStream_t stream) {
     if (segments <= 0 || rows <= 0) return 0;
     if (heads <= 0 || heads > 65535 || V <= 0 || !(cap > 0.f)) return (int)hipErrorInvalidValue;
-    mlstm_rows_kernel<<<rows, 256, 0, stream>>>(zi, ldi, zf, ldf, bi, bf, v, ldv, decay, step, vx, heads, V, cap);
+    if (single_rows) {
+        mlstm_rows_kernel<true><<<rows, 256, 0, stream>>>(zi, ldi, zf, ldf, bi, bf, v, ldv, decay, step, vx, heads, V, cap, top, state,
+                                                          slot_stride, seg_start, state_slots, segments);
+        return CISR_LAUNCH_CHECK();
+    }
+    mlstm_rows_kernel<false><<<rows, 256, 0, stream>>>(zi, ldi, zf, ldf, bi, bf, v, ldv, decay, step, vx, heads, V, cap, top, state,
+                                                       slot_stride, seg_start, state_slots, segments);
     int err = CISR_LAUNCH_CHECK();
     if (err) return err;
     mlstm_walk_kernel<<<dim3(segments, heads), 64, 0, stream>>>(decay, step, top, state, slot_stride, seg_start, state_slots, heads);

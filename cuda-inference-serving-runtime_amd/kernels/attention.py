@@ -387,6 +387,14 @@ def talking_splits(tiles, span):
     return int(max(1, min(-(-256 // max(tiles, 1)), steps // 4, 8)))
 
 
+def talking_row_splits(rows, span):
+    """Blocks that share a row's keys in the exact form of the attention with mixed scores (one block a row otherwise):
+    steps of few rows split the keys until the launch has about a block for every compute unit, each keeping at least
+    two tiles of 64 keys."""
+    tiles = max(1, -(-span // 64))
+    return int(max(1, min(256 // max(rows, 1), tiles // 2, 16)))
+
+
 def talking_attention(ctx, q, kcache, vcache, view, out, heads, kv_heads, vdim, pad, mix, scale, temp=None, sink=None,
                       window=None, chunk=None, gate=None):
     """out[r] = attention of row r over its request's cached keys where the scores of all heads of a row are mixed
@@ -408,6 +416,13 @@ def talking_attention(ctx, q, kcache, vcache, view, out, heads, kv_heads, vdim, 
                                     view.page_size, mix, scale, temp=temp, sink=sink, window=window, chunk=chunk, gate=gate,
                                     splits=splits, workspace=workspace)
         return out
+    rows = out.shape[0]
+    splits = talking_row_splits(rows, min(ctx.span_hint, chunk or window or ctx.span_hint))
+    workspace = None
+    if splits > 1:
+        workspace = (ctx.buffer("tattn.part_o", (rows * heads * splits * vdim,), torch.float32),
+                     ctx.buffer("tattn.part_ml", (rows * heads * splits * 2,), torch.float32))
     ops.attention_talking(q, q.stride(0), kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out, heads, kv_heads, vdim, pad,
-                          view.page_size, mix, scale, temp=temp, sink=sink, window=window, chunk=chunk, gate=gate)
+                          view.page_size, mix, scale, temp=temp, sink=sink, window=window, chunk=chunk, gate=gate, splits=splits,
+                          workspace=workspace)
     return out

@@ -69,7 +69,7 @@ def _declare(h):
         "cisr_gemm_skinny_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
         "cisr_gemm_wide_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p, C.c_longlong, p],
         "cisr_gemm_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
-        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, i, i, f, f, p],
+        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, i, i, f, f, p, p],
         "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
         "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
         "cisr_head_gate": [p, p, i, p, i, i, i, i, i, p],
@@ -86,7 +86,7 @@ def _declare(h):
         "cisr_embedding_pairs": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, f, i, ll, ll, i, i, i, p],
         "cisr_gate_post_norm": [p, p, i, p, p, i, p, p, p, i, i, f, f, i, p],
         "cisr_whole_norm_rope_scatter": [p, i, p, p, p, p, p, p, p, i, i, p, p, p, i, i, i, i, i, i, i, f, i, i, i, i, p],
-        "cisr_attn_talking": [p, i, p, p, p, p, p, p, p, p, p, i, p, i, i, i, i, i, i, i, i, i, f, i, p],
+        "cisr_attn_talking": [p, i, p, p, p, p, p, p, p, p, p, i, p, i, i, i, i, i, i, i, i, i, f, i, p, p, i, p],
         "cisr_experts_route": [p, i, p, p, p, i, i, i, i, p, p, p],
         "cisr_experts_gemm": [p, i, p, p, p, i, i, p, i, i, i, i, i, i, i, p],
         "cisr_experts_rows": [p, i, p, p, i, p, i, i, i, i, i, i, i, p],
@@ -373,15 +373,21 @@ LIBRARY_GATED_MIN_ROWS, LIBRARY_GATED_MIN_BYTES = 33, 64 << 20
 
 
 def attention_talking(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, vdim, pad, page_size,
-                      mix, scale, temp=None, sink=None, window=None, chunk=None, gate=None):
+                      mix, scale, temp=None, sink=None, window=None, chunk=None, gate=None, splits=1, workspace=None):
     """Attention whose scores are mixed over the heads before the softmax: s_h = sum_g mix[h, g] temp[g] scale (q_g . k),
     weights exp(s_h) / (exp(sink_h) + sum over the visible keys), out_h = sum w_h v of the head's key/value head, times
     sigmoid(gate) element by element.  A row at position p sees the keys of its block of `chunk` positions up to itself
     (or the last `window`, or all).  q [T, >= heads * pad] and the pages hold heads of `pad` coordinates, the rest zero;
     out [T, heads * vdim]; mix float [heads, heads], temp and sink float [heads] or None; gate a float view
-    [T, heads * vdim] or None."""
+    [T, heads * vdim] or None.  `splits` > 1: that many blocks share a row's keys and leave their sums in `workspace` =
+    (float [T * heads * splits * vdim], float [T * heads * splits * 2]) for a merge kernel behind them."""
     rows = out.shape[0]
     pages = kcache.shape[0]
+    po = pm = None
+    if splits > 1:
+        if workspace is None or workspace[0].numel() < rows * heads * splits * vdim or workspace[1].numel() < rows * heads * splits * 2:
+            raise KernelError("attention_talking: split keys need a workspace for their sums")
+        po, pm = _dev(workspace[0], "part_o", torch.float32), _dev(workspace[1], "part_ml", torch.float32)
     gp, ldg = None, 0
     if gate is not None:
         if gate.dtype != torch.float32 or tuple(gate.shape) != (rows, heads * vdim) or gate.stride(1) != 1 or not gate.is_cuda:
@@ -397,7 +403,8 @@ def attention_talking(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
                                    None if temp is None else _dev(temp, "temp", torch.float32, (heads,)),
                                    None if sink is None else _dev(sink, "sink", torch.float32, (heads,)), gp, ldg,
                                    _dev(out, "out", None, (rows, heads * vdim)), rows, heads, kv_heads, vdim, pad, page_size, width,
-                                   int(window or 0), int(chunk or 0), float(scale), _storage(out, "out"), _stream()), "attention_talking")
+                                   int(window or 0), int(chunk or 0), float(scale), int(splits), po, pm, _storage(out, "out"), _stream()),
+           "attention_talking")
     return out
 
 
@@ -1015,6 +1022,14 @@ def gemm_for_norm(a, w, out, make_buffer, scratch=None):
     return gemm(a, w, out, scratch=scratch)
 
 
+class Biased:
+    """Float rows [T, N] that still lack a bias a column (float [N]): a product's result whose bias is left to the kernel
+    that reads it next (post_norm_add adds it on the way)."""
+
+    def __init__(self, rows, bias):
+        self.rows, self.bias = rows, bias
+
+
 def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
     """x += mult * rmsnorm(y) * weight, in place (all float, [T, H]).  With `second` = (y2, w1, w2) the row that is
     normed is (rmsnorm(y) w1 + rmsnorm(y2) w2) / 2: two sublayers side by side; with `second` = (y2, c1, c2), two
@@ -1024,6 +1039,9 @@ def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
     y (and y2) may be a Partials of [T, H]: its slices are added on the way."""
     rows, dim = x.shape
     xp = _dev(x, "x", torch.float32)
+    bias_p = None
+    if isinstance(y, Biased):          # (y + bias, added as the rows are read)
+        bias_p, y = _dev(y.bias, "bias of y", torch.float32, (dim,)), y.rows
 
     def operand(t, name):
         if isinstance(t, Partials):
@@ -1050,7 +1068,7 @@ def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
         np_ = None if nw is None else _dev(nw, "following weight", torch.float32, (dim,))
         op, odt = _dev(out, "following out", None, (rows, dim)), _storage(out, "following out")
     _check(lib().cisr_post_norm_add(xp, yp, ap, bp, w2p, wp, rows, dim, float(eps), float(mult), np_, float(neps), op, odt,
-                                    slices_a, slices_b, ca, cb, _stream()), "post_norm_add")
+                                    slices_a, slices_b, ca, cb, bias_p, _stream()), "post_norm_add")
     return x
 
 
@@ -1244,7 +1262,7 @@ def _rec():
             "cisr_delta_scan": [p, i, p, i, p, i, p, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
             "cisr_unit_heads": [p, i, i, i, i, i, f, f, p],
             "cisr_mingru_scan": [p, i, p, p, p, i, p, p, p, i, i, i, i, p, i, i, p],
-            "cisr_mlstm_gates": [p, i, p, i, p, p, p, i, p, p, p, p, p, ll, p, p, i, i, i, i, f, p],
+            "cisr_mlstm_gates": [p, i, p, i, p, p, p, i, p, p, p, p, p, ll, p, p, i, i, i, i, f, i, p],
             "cisr_mlstm_finish": [p, p, p, i, p, p, i, i, i, f, f, i, p],
         }
         for name, args in sig.items():
@@ -1679,12 +1697,13 @@ def experts_gemm(a, w, pair_of_pos, tile_expert, out, top=0, scatter=False, act=
     return out
 
 
-def mlstm_gates(zi, zf, bias_i, bias_f, v, decay, step, top, vx, top_state, seg_start, state_slots, heads, vdim, cap):
+def mlstm_gates(zi, zf, bias_i, bias_f, v, decay, step, top, vx, top_state, seg_start, state_slots, heads, vdim, cap, single_rows=False):
     """The operands of the matrix memory's scan from the projections' float results: log gates i = cap tanh((zi + bi) /
     cap), f = logsigmoid(cap tanh((zf + bf) / cap)) (zi, zf float views [T, heads]); along every segment's rows the
     running maximum m' = max(f + m, i), from `top_state`[slot, head] and back into it; decay = exp(f + m - m'), step =
     exp(i - m') and top = m', float [T, heads]; vx [T, heads * (vdim + 1)] = the values v (a float view [T, heads *
-    vdim]) with a column of ones a head."""
+    vdim]) with a column of ones a head.  `single_rows`: every segment has one row (row t is segment t; rows past the
+    segments are padding): one kernel makes the gates and moves the maxima on."""
     T = v.shape[0]
     segments = state_slots.shape[0]
     ip, ldi = _rows_of(zi, "zi", heads)
@@ -1696,8 +1715,8 @@ def mlstm_gates(zi, zf, bias_i, bias_f, v, decay, step, top, vx, top_state, seg_
                                    vp, ldv, _dev(decay, "decay", torch.float32, (T, heads)), _dev(step, "step", torch.float32, (T, heads)),
                                    _dev(top, "top", torch.float32, (T, heads)), _dev(vx, "vx", torch.float32, (T, heads * (vdim + 1))),
                                    top_state.data_ptr(), top_state.stride(0), _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
-                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), T, segments, heads, vdim, float(cap), _stream()),
-           "mlstm_gates")
+                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), T, segments, heads, vdim, float(cap), int(bool(single_rows)),
+                                   _stream()), "mlstm_gates")
 
 
 def mlstm_finish(o, top, gate, weight, out, heads, vdim, eps, floor=1e-6):

@@ -522,8 +522,9 @@ class TalkingAttention(Mixer):
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
 
-    def output(self, h, ctx, site, scale=1.0):
-        """The mixer's result times `scale`, float [T, hidden], without the residual sum."""
+    def output(self, h, ctx, site):
+        """The mixer's result, float [T, hidden] (an ops.Biased where the output projection has a bias), without the
+        residual sum."""
         T = h.shape[0]
         nh, nkv, D, V, pad = self.heads, self.kv_heads, self.dim, self.vdim, self.pad
         gid, kcache, vcache = ctx.cache.pages_of_site(site)
@@ -539,7 +540,7 @@ class TalkingAttention(Mixer):
         kernel.talking_attention(ctx, q, kcache, vcache, view, act, nh, nkv, V, pad, self.talk, self.scale, temp=self.temp, sink=self.sink,
                                  chunk=self.chunk, gate=proj[:, first:first + nh * V] if self.has_gate else None)
         y = ops.gemm(act, self.w_out, ctx.buffer("tattn.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
-        return y if self.b_out is None else ops.bias_add(y, self.b_out)
+        return y if self.b_out is None else ops.Biased(y, self.b_out)       # (the kernel that adds the result adds the bias)
 
     def forward(self, h, residual, ctx, site, norm=None):
         from .block import add_sublayer

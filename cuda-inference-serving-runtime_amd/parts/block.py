@@ -309,6 +309,8 @@ class PostNormBlock(Part):
 
     def _sum_and_norm(self, x, h, result, which, sub, norm, ctx):
         """x <- norm(alpha x + gate * result) in place; returns the new rows in the activations' type."""
+        if isinstance(result, ops.Biased):
+            result = ops.bias_add(result.rows, result.bias)
         if isinstance(result, ops.Partials):
             raise TypeError("a sublayer of this arrangement gives finished rows (or weighted rows), no partial sums")
         gate = bias = None

@@ -148,7 +148,7 @@ class DenseMLP(FeedForward):
         """The feed-forward's result, float [T, hidden], without the residual sum."""
         if self.bias:
             y = ops.gemm(self._activations(h, ctx), self.w_down, ctx.buffer("ffn.out", (h.shape[0], self.hidden), torch.float32), scratch=ctx.scratch)
-            return ops.bias_add(y, self.b_down)
+            return ops.Biased(y, self.b_down)          # (the kernel that adds the result adds the bias)
         return ctx.product_for_norm(self._activations(h, ctx), self.w_down, "ffn.out")
 
     def forward(self, h, residual, ctx, norm=None):

@@ -376,7 +376,7 @@ class MatrixMemory(Mixer):
         vx = ctx.buffer("mm.vx", (T, nh * C), torch.float32)
         gates = 2 * K + 2 * W
         ops.mlstm_gates(proj[:, gates:gates + nh], proj[:, gates + nh:gates + 2 * nh], self.bias_i, self.bias_f, proj[:, 2 * K:2 * K + W],
-                        decay, step, top, vx, state[:, K * C:], ctx.seg_start, ctx.state_slots, nh, V, self.cap)
+                        decay, step, top, vx, state[:, K * C:], ctx.seg_start, ctx.state_slots, nh, V, self.cap, single_rows=ctx.decode_only)
         o = ctx.buffer("mm.o", (T, nh * C), torch.float32)
         _scan(ctx, "mm", proj[:, :K], proj[:, K:2 * K], vx, decay, o, state, nh, R, C, step=step, q_scale=R ** -0.5)
         act = ops.mlstm_finish(o, top, proj[:, 2 * K + W:2 * K + 2 * W], self.norm_weight, ctx.buffer("mm.act", (T, W), ctx.dtype),

@@ -137,6 +137,13 @@ def test_attention_with_mixed_scores_alone(dtype, heads, kv_heads, dim, vdim, ch
     if gate:
         want = want * sigmoid(rounded(gates[:, :heads * vdim], "float32"))
     close(out.float().cpu().numpy(), want, 2e-5 if dtype == "float32" else 1.5e-2)
+    # five blocks along a row's keys, merged (more blocks than some rows have tiles of keys)
+    out.fill_(float("nan"))
+    work = (torch.full((rows * heads * 5 * vdim,), float("nan"), device="cuda"), torch.full((rows * heads * 5 * 2,), float("nan"), device="cuda"))
+    ops.attention_talking(dev(q.reshape(rows, -1), td), heads * pad, dev(K, td), dev(V, td), ints(tables), ints(seg_of_row), ints(positions), out,
+                          heads, kv_heads, vdim, pad, page_size, dev(mix), 0.2, temp=dev(temp), sink=dev(sinks) if sink else None,
+                          window=window, chunk=chunk, gate=dev(gates)[:, :heads * vdim] if gate else None, splits=5, workspace=work)
+    close(out.float().cpu().numpy(), want, 2e-5 if dtype == "float32" else 1.5e-2)
     if ops.talking_tiles_ok(td, heads, kv_heads, vdim, pad, page_size):
         # the same rows as tiles of 16 on the matrix cores, the tiles in another order and padded with empty ones
         from runtime.kernels.attention import fill_tasks
@@ -183,7 +190,7 @@ def test_matrix_memory_over_segments_with_states_carried_and_slots_used_again(he
         vx = torch.empty(T, heads * C, device="cuda")
         g0 = 2 * K + 2 * W
         ops.mlstm_gates(dp[:, g0:g0 + heads], dp[:, g0 + heads:g0 + 2 * heads], dev(bi), dev(bf), dp[:, 2 * K:2 * K + W], decay, step, top, vx,
-                        state[:, K * C:], ints(start), ints(slots), heads, vdim, cap)
+                        state[:, K * C:], ints(start), ints(slots), heads, vdim, cap, single_rows=all(c == 1 for c in counts))
         o = torch.full((T, heads * C), float("nan"), device="cuda")
         p = 0 if all(c == 1 for c in counts) else piece
         carry = None
