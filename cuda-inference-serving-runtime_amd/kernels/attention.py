@@ -388,11 +388,11 @@ def talking_splits(tiles, span):
 
 
 def talking_row_splits(rows, span):
-    """Blocks that share a row's keys in the exact form of the attention with mixed scores (one block a row otherwise):
-    steps of few rows split the keys until the launch has about a block for every compute unit, each keeping at least
-    two tiles of 64 keys."""
+    """Blocks that share a row's keys in the exact form of the attention with mixed scores (one block a row otherwise).
+    A block takes about 10 us a tile of 64 keys (its loads wait for each other), so steps of few rows give every tile
+    a block of its own until the launch has about four blocks a compute unit."""
     tiles = max(1, -(-span // 64))
-    return int(max(1, min(256 // max(rows, 1), tiles // 2, 16)))
+    return int(max(1, min(1024 // max(rows, 1), tiles, 32)))
 
 
 def talking_attention(ctx, q, kcache, vcache, view, out, heads, kv_heads, vdim, pad, mix, scale, temp=None, sink=None,
