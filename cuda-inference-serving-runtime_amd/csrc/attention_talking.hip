@@ -114,15 +114,23 @@ attn_talking_kernel(TalkArgs p) {
             for (int g0 = 0; g0 < group; g0 += 4) {
                 float dot[4] = {0.f, 0.f, 0.f, 0.f};
                 const float* q0 = qs + (size_t)(c * group + g0) * pad;
-                for (int d = 0; d < pad; d += 8) {
-                    float kv[8];
-                    load8(kr + d, kv);
+                for (int d0 = 0; d0 < pad; d0 += 64) {             // 64 coordinates a trip: eight loads on their way together
+                    float kv[8][8];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        if (g0 + u < group) {
-                            const float* qh = q0 + u * pad + d;
+                    for (int w = 0; w < 8; ++w) {
+                        if (d0 + 8 * w < pad) load8(kr + d0 + 8 * w, kv[w]);
+                    }
 #pragma unroll
-                            for (int i = 0; i < 8; ++i) dot[u] += qh[i] * kv[i];
+                    for (int w = 0; w < 8; ++w) {
+                        const int d = d0 + 8 * w;
+                        if (d >= pad) continue;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            if (g0 + u < group) {
+                                const float* qh = q0 + u * pad + d;
+#pragma unroll
+                                for (int i = 0; i < 8; ++i) dot[u] += qh[i] * kv[w][i];
+                            }
                         }
                     }
                 }
@@ -163,15 +171,23 @@ attn_talking_kernel(TalkArgs p) {
             float a = acc[e] * alpha[h];
             const float* wr = pw + h * TK_KEYS;
             if (by8) {
-                for (int j = 0; j < TK_KEYS; j += 8) {
+                // the tile's eight groups of eight keys: all loads on their way before the first is used
+                float vv[8][8];
+                bool there[8];
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    const int j = 8 * w;
                     int page = -1;
 #pragma unroll
                     for (int u = 0; u < 8; ++u) page = max(page, pg[j + u]);      // (eight keys from a multiple of eight: one page)
-                    if (page < 0) continue;
-                    float vv[8];
-                    load8(vc + (((size_t)page * G + c) * pad + d) * P + po[j], vv);
+                    there[w] = page >= 0;
+                    if (there[w]) load8(vc + (((size_t)page * G + c) * pad + d) * P + po[j], vv[w]);
+                }
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) a += wr[j + u] * vv[u];
+                for (int w = 0; w < 8; ++w) {
+                    if (!there[w]) continue;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) a += wr[8 * w + u] * vv[w][u];
                 }
             } else {
                 for (int j = 0; j < TK_KEYS; ++j)
@@ -241,6 +257,18 @@ static int launch_talking(const TalkArgs& a, int rows, hipStream_t stream) {
     const size_t lds = talking_lds(a.heads, a.pad);
     const int per = (a.heads * a.vdim + 255) / 256;
     const dim3 grid(rows, a.splits);
+    if (lds > 48 * 1024) {                                       // (many heads: the limit of dynamic LDS above the default, once a kernel)
+        static bool raised = false;
+        if (!raised) {
+            const void* kernels[] = {(const void*)attn_talking_kernel<T, 2>, (const void*)attn_talking_kernel<T, 4>, (const void*)attn_talking_kernel<T, 8>,
+                                     (const void*)attn_talking_kernel<T, 16>, (const void*)attn_talking_kernel<T, 32>};
+            for (const void* k : kernels) {
+                const int err = (int)hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (err) return err;
+            }
+            raised = true;
+        }
+    }
 #define TALK(E) attn_talking_kernel<T, E><<<grid, 256, lds, stream>>>(a)
     if (per <= 2) TALK(2);
     else if (per <= 4) TALK(4);
@@ -263,7 +291,7 @@ extern "C" int cisr_attn_talking(const void* q, int q_row_stride, const void* kc
     if (rows <= 0) return 0;
     if (splits < 1 || splits > 65535 || heads > 65535 || (splits > 1 && (!part_o || !part_ml))) return (int)hipErrorInvalidValue;
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || pad <= 0 || pad % 8 || vdim <= 0 || vdim > pad || page_size <= 0 ||
-        !mix || talking_lds(heads, pad) > 64 * 1024 || q_row_stride < heads * pad || (gate && ldg < heads * vdim))
+        !mix || talking_lds(heads, pad) > 160 * 1024 || q_row_stride < heads * pad || (gate && ldg < heads * vdim))
         return (int)hipErrorInvalidValue;
     const TalkArgs a = {q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, mix, temp, sink, gate, ldg, out,
                         heads, kv_heads, vdim, pad, page_size, width, window, chunk, scale, splits, part_o, part_ml};

@@ -145,6 +145,89 @@ route_scored_kernel(const float* __restrict__ logits, int ld, const float* __res
     }
 }
 
+// The same routing with a wave a row (routers of at most 512 outputs): lane l holds the outputs l, l + 64, ...; the
+// maximum, the sum, a group's best and every choice are reductions over the wave, so a step of few rows does not wait
+// for one thread's chain of exponentials.  The lowest index wins a tie, as above.
+#define ROUTE_PER_LANE 8
+__global__ void __launch_bounds__(256)
+route_scored_wave_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int* __restrict__ chosen,
+                         float* __restrict__ weights, int rows, int outputs, int top, int groups, int keep) {
+    const int row = blockIdx.x * 4 + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    if (row >= rows) return;
+    const float* lr = logits + (size_t)row * ld;
+    float z[ROUTE_PER_LANE], largest = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+        const int e = lane + WAVE * i;
+        z[i] = e < outputs ? lr[e] : -INFINITY;
+        largest = fmaxf(largest, z[i]);
+    }
+    largest = wave_max(largest);
+    float den = 0.f, s[ROUTE_PER_LANE], c[ROUTE_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) { s[i] = lane + WAVE * i < outputs ? expf(z[i] - largest) : 0.f; den += s[i]; }
+    den = wave_sum(den);
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+        const int e = lane + WAVE * i;
+        s[i] /= den;
+        c[i] = e < outputs ? s[i] + (correction ? correction[e] : 0.f) : -INFINITY;      // -inf: not there, dropped or taken
+    }
+    // the best (value, lowest index) over the wave among this lane's candidates `v`
+    auto best_of = [&](const float (&v)[ROUTE_PER_LANE], float& bv, int& be) {
+        bv = -INFINITY; be = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+            const int e = lane + WAVE * i;
+            if (e < outputs && (v[i] > bv || (v[i] == bv && e < be))) { bv = v[i]; be = e; }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, WAVE);
+            const int oe = __shfl_xor(be, off, WAVE);
+            if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+        }
+    };
+    if (groups > 0) {
+        const int per = outputs / groups;
+        unsigned long long kept = 0ull;
+        for (int k = 0; k < keep; ++k) {
+            // the group, not kept yet, whose largest choice score is largest (the lowest group wins a tie): a group's
+            // largest score is the score of its best member, and of two equal ones the lower index lies in the lower group
+            float v[ROUTE_PER_LANE];
+#pragma unroll
+            for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+                const int e = lane + WAVE * i;
+                v[i] = (e < outputs && !((kept >> (e / per)) & 1ull)) ? c[i] : -INFINITY;
+            }
+            float bv; int be;
+            best_of(v, bv, be);
+            int g = be / per;
+            if (bv == -INFINITY) {                               // (every candidate at minus infinity: the lowest group not kept)
+                g = 0;
+                while ((kept >> g) & 1ull) ++g;
+            }
+            kept |= 1ull << g;
+        }
+#pragma unroll
+        for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+            const int e = lane + WAVE * i;
+            if (e < outputs && !((kept >> (e / per)) & 1ull)) c[i] = -INFINITY;
+        }
+    }
+    for (int k = 0; k < top; ++k) {
+        float bv; int be;
+        best_of(c, bv, be);
+        float share = 0.f;
+#pragma unroll
+        for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+            if (lane + WAVE * i == be) { share = s[i]; c[i] = -INFINITY; }
+        }
+        share = wave_sum(share);                                 // (one lane holds it)
+        if (lane == 0) { chosen[(size_t)row * top + k] = be; weights[(size_t)row * top + k] = share; }
+    }
+}
+
 // `experts` of the router's `outputs` have matrices (the first ones): only their pairs are arranged into tiles.
 extern "C" int cisr_experts_route_scored(const float* logits, int ld, const float* correction, int* chosen, float* weights, int rows,
                                          int outputs, int experts, int top, int groups, int keep, int max_tiles, int* pair_of_pos,
@@ -155,7 +238,11 @@ extern "C" int cisr_experts_route_scored(const float* logits, int ld, const floa
         groups > 64 || (groups > 0 && (outputs % groups || keep <= 0 || keep > groups || keep * (outputs / groups) < top)) ||
         (arrange && (!tile_expert || (long long)max_tiles * EX_TILE < (long long)rows * top + (long long)experts * (EX_TILE - 1))))
         return (int)hipErrorInvalidValue;
-    route_scored_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(logits, ld, correction, chosen, weights, rows, outputs, top, groups, keep);
+    // steps of few rows: a wave a row; many rows keep a thread a row (the GPU is full either way, and a thread's chain is short beside the step)
+    if (outputs <= WAVE * ROUTE_PER_LANE && rows <= 4096)
+        route_scored_wave_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(logits, ld, correction, chosen, weights, rows, outputs, top, groups, keep);
+    else
+        route_scored_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(logits, ld, correction, chosen, weights, rows, outputs, top, groups, keep);
     int err = CISR_LAUNCH_CHECK();
     if (err || !arrange) return err;
     arrange_kernel<<<1, 1024, 3 * experts * sizeof(int), stream>>>(chosen, rows * top, experts, max_tiles, pair_of_pos, tile_expert);

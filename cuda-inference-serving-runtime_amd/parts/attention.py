@@ -468,6 +468,7 @@ class TalkingAttention(Mixer):
         self.bias, self.has_temp, self.has_sink, self.has_gate, self.value_norm = tuple(bias), bool(temp), bool(sink), bool(gate), bool(value_norm)
         self.names = {**self.NAMES, **(names or {})}
         self.w_in = self.w_out = self.b_in = self.b_out = self.q_weight = self.k_weight = self.talk = self.temp = self.sink = None
+        self.rider, self.rider_rows = None, 0
 
     def _tensor(self, which):
         return f"{self.name}.{self.names[which]}"
@@ -500,11 +501,9 @@ class TalkingAttention(Mixer):
     def bind(self, tensors, dtype):
         t = self._tensor
         inputs = ("q", "k", "v") + (("g",) if self.has_gate else ())
-        parts = [matrix_operand(tensors[t(p)], dtype) for p in inputs]
-        rows = sum(p.shape[0] for p in parts)
-        if rows % 8:      # rows of the fused projection are a multiple of 8: zero rows at the end
-            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
-        self.w_in = torch.cat(parts, dim=0).contiguous()
+        parts = self.w_own = [matrix_operand(tensors[t(p)], dtype) for p in inputs]
+        self.own_rows = sum(p.shape[0] for p in parts)
+        self._join()
         self.w_out = matrix_operand(tensors[t("o")], dtype)
 
         def f32(x):
@@ -519,6 +518,19 @@ class TalkingAttention(Mixer):
         self.temp = f32(tensors[t("temp")]) if self.has_temp else None
         self.sink = f32(tensors[t("sink")]) if self.has_sink else None
 
+    def _join(self, extra=None):
+        parts = list(self.w_own) + ([] if extra is None else [extra])
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:      # rows of the fused projection are a multiple of 8: zero rows at the end
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+
+    def ride(self, weight):
+        """Further rows for the input product (a neighbour that reads the same h); their float results are `rider`
+        after `output`."""
+        self.rider_rows = weight.shape[0]
+        self._join(weight)
+
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
 
@@ -532,6 +544,7 @@ class TalkingAttention(Mixer):
         cos, sin = self.position.tables()
         # queries, keys and values before their norms are float (the norms' statistics are), and so is the gate
         proj = ops.gemm(h, self.w_in, ctx.buffer("tattn.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        self.rider = proj[:, self.own_rows:self.own_rows + self.rider_rows] if self.rider_rows else None
         q = ctx.buffer("tattn.q", (T, nh * pad), ctx.dtype)
         ops.whole_norm_rope_scatter(proj, self.q_weight, self.k_weight, ctx.positions, view.slots, cos, sin, q, kcache, vcache,
                                     nh, nkv, D, V, pad, view.page_size, self.eps, bias=self.b_in, split_half=True, value_norm=self.value_norm)

@@ -365,11 +365,17 @@ class MatrixMemory(Mixer):
         self.norm_weight = _float(tensors[t("norm")])
         self.bias_i, self.bias_f = _float(tensors[t("i") + ".b"]), _float(tensors[t("f") + ".b"])
 
-    def output(self, h, ctx, site):
+    def input_weight(self):
+        """The matrix of the input product, for a neighbour that reads the same h and makes both products as one (its
+        float results then come back as `proj` of `output`)."""
+        return self.w_in
+
+    def output(self, h, ctx, site, proj=None):
         T = h.shape[0]
         nh, R, V = self.heads, self.dim, self.vdim
         K, W, C = nh * R, nh * V, V + 1
-        proj = ops.gemm(h, self.w_in, ctx.buffer("mm.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        if proj is None:
+            proj = ops.gemm(h, self.w_in, ctx.buffer("mm.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
         state = ctx.cache.state_storage[site]
         state = state.view(state.shape[0], -1)
         decay, step, top = (ctx.buffer("mm." + n, (T, nh), torch.float32) for n in ("decay", "step", "top"))
@@ -425,6 +431,11 @@ class SideBySide(Mixer):
         for m in self.mixers():
             m.bind(tensors, dtype)
         self.out_weights = [_float(tensors[n]) for n in self.out_names]
+        # both read the same h: where the first takes further rows into its input product and the second can be handed
+        # its projection, the two products are one
+        self.joined = self.scales is not None and hasattr(self.first, "ride") and hasattr(self.second, "input_weight")
+        if self.joined:
+            self.first.ride(self.second.input_weight())
 
     def prepare(self, device, dtype):
         for m in self.mixers():
@@ -433,7 +444,9 @@ class SideBySide(Mixer):
     def output(self, h, ctx, site):
         from .block import NormedMean, ScaledSum
         if self.scales is not None:
-            return ScaledSum(self.first.output(h, ctx, site), self.scales[0], self.second.output(h, ctx, site), self.scales[1])
+            first = self.first.output(h, ctx, site)
+            second = self.second.output(h, ctx, site, proj=self.first.rider) if self.joined else self.second.output(h, ctx, site)
+            return ScaledSum(first, self.scales[0], second, self.scales[1])
         return NormedMean(self.first.output(h, ctx, site), self.out_weights[0], self.second.output(h, ctx, site),
                           self.out_weights[1], self.eps)
 

@@ -66,7 +66,8 @@ def rounded(a, dtype):
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim, chunk, window, page_size, sink, gate", [
     (4, 2, 24, 16, 20, None, 16, True, True), (1, 1, 10, 24, 1, None, 16, True, False), (20, 4, 64, 64, 100, None, 8, True, True),
     (3, 3, 16, 40, None, None, 16, False, True), (6, 2, 8, 8, None, 33, 4, True, False), (40, 8, 32, 48, 70, None, 16, True, True),
-    (16, 4, 128, 128, 128, None, 16, True, True), (32, 8, 96, 80, None, None, 32, False, True), (6, 3, 128, 80, 64, None, 16, True, False)])
+    (16, 4, 128, 128, 128, None, 16, True, True), (32, 8, 96, 80, None, None, 32, False, True), (6, 3, 128, 80, 64, None, 16, True, False),
+    (64, 16, 128, 64, 50, None, 16, True, True), (12, 12, 136, 160, 90, None, 16, True, True)])
 def test_attention_with_mixed_scores_alone(dtype, heads, kv_heads, dim, vdim, chunk, window, page_size, sink, gate):
     """Rows of three requests (a long portion, a single token far into its sequence, a sequence's first tokens) against
     the plain sums; the pages lie scattered, pages before a row's block are not there (-1 in the table).  One query and
@@ -230,11 +231,11 @@ def test_matrix_memory_over_segments_with_states_carried_and_slots_used_again(he
 
 
 @pytest.mark.parametrize("rows, experts, identity, top, groups", [(1, 2, 0, 2, None), (9, 6, 2, 3, (4, 2)), (300, 14, 2, 4, (4, 2)), (70, 3, 1, 2, (2, 1)),
-                                                                  (33, 5, 0, 1, None), (40, 4, 4, 3, (2, 2))])
+                                                                  (33, 5, 0, 1, None), (40, 4, 4, 3, (2, 2)), (4500, 6, 2, 3, (4, 2)), (50, 130, 6, 5, (8, 3))])
 def test_routing_by_scores_with_a_correction_and_groups(rows, experts, identity, top, groups):
     """The choice and the weights against the plain routing (corrections that are negative as well, so that a dropped
     group must count as minus infinity and not as zero); the layout by expert holds every pair of an expert with
-    matrices once and no pair of an identity expert."""
+    matrices once and no pair of an identity expert.  Steps of few rows route a wave a row, many rows a thread a row."""
     from runtime.kernels import ops
     rng = np.random.default_rng(rows + experts)
     n = experts + identity
