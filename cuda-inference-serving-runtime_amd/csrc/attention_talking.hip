@@ -66,6 +66,13 @@ attn_talking_kernel(TalkArgs p) {
     float acc[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) acc[e] = 0.f;
+    // Which output a thread's e-th accumulator is: coordinate (tid + 256 e) of the row as it lies in memory; or, where
+    // the sizes allow (value heads that divide 256 and head counts that divide by 256 / vdim), one coordinate d of
+    // consecutive heads, so that heads of one group follow each other and share the loads of their values.
+    const int lanes_of_d = 256 / p.vdim;
+    const bool packed = 256 % p.vdim == 0 && H % lanes_of_d == 0 && H / lanes_of_d <= E;
+    const int heads_here = packed ? H / lanes_of_d : 0;
+    auto owned = [&](int e) { return packed ? (e < heads_here ? ((tid / p.vdim) * heads_here + e) * p.vdim + tid % p.vdim : n_out) : tid + 256 * e; };
     int begin = 0, end = 0;
     if (seg >= 0) {
         const int pos = p.positions[row];
@@ -82,7 +89,7 @@ attn_talking_kernel(TalkArgs p) {
             return;
         }
 #pragma unroll
-        for (int e = 0; e < E; ++e) { const int i = tid + 256 * e; if (i < n_out) store_f32(out + i, 0.f); }
+        for (int e = 0; e < E; ++e) { const int i = owned(e); if (i < n_out) store_f32(out + i, 0.f); }
         return;
     }
     const T* qr = (const T*)p.q + (size_t)row * p.q_row_stride;
@@ -163,25 +170,30 @@ attn_talking_kernel(TalkArgs p) {
         }
         __syncthreads();
         // (4) the values
+        float vv[8][8];
+        bool there[8];
+        int c_held = -1, d_held = -1;                            // the key head and coordinate whose values vv holds
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int i = tid + 256 * e;
+            const int i = owned(e);
             if (i >= n_out) continue;
             const int h = i / p.vdim, d = i % p.vdim, c = h / group;
             float a = acc[e] * alpha[h];
             const float* wr = pw + h * TK_KEYS;
             if (by8) {
-                // the tile's eight groups of eight keys: all loads on their way before the first is used
-                float vv[8][8];
-                bool there[8];
+                // the tile's eight groups of eight keys: all loads on their way before the first is used; the values
+                // stay for the next accumulator if that is a head of the same group
+                if (c != c_held || d != d_held) {
+                    c_held = c; d_held = d;
 #pragma unroll
-                for (int w = 0; w < 8; ++w) {
-                    const int j = 8 * w;
-                    int page = -1;
+                    for (int w = 0; w < 8; ++w) {
+                        const int j = 8 * w;
+                        int page = -1;
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) page = max(page, pg[j + u]);      // (eight keys from a multiple of eight: one page)
-                    there[w] = page >= 0;
-                    if (there[w]) load8(vc + (((size_t)page * G + c) * pad + d) * P + po[j], vv[w]);
+                        for (int u = 0; u < 8; ++u) page = max(page, pg[j + u]);      // (eight keys from a multiple of eight: one page)
+                        there[w] = page >= 0;
+                        if (there[w]) load8(vc + (((size_t)page * G + c) * pad + d) * P + po[j], vv[w]);
+                    }
                 }
 #pragma unroll
                 for (int w = 0; w < 8; ++w) {
@@ -200,7 +212,7 @@ attn_talking_kernel(TalkArgs p) {
     if (S > 1) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int i = tid + 256 * e;
+            const int i = owned(e);
             if (i >= n_out) continue;
             const int h = i / p.vdim, d = i % p.vdim;
             p.part_o[(((size_t)row * H + h) * S + split) * p.vdim + d] = acc[e];
@@ -213,7 +225,7 @@ attn_talking_kernel(TalkArgs p) {
     }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const int i = tid + 256 * e;
+        const int i = owned(e);
         if (i >= n_out) continue;
         const float l = run_l[i / p.vdim];
         float v = l > 0.f ? acc[e] / l : 0.f;

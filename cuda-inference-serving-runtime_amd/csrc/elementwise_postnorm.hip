@@ -176,7 +176,9 @@ whole_norm_rope_scatter_kernel(const float* __restrict__ proj, int ld, const flo
         const float co = cr[pair], si = sr[pair];
         return second ? own * co + other * si : own * co - other * si;
     };
-    for (int i = threadIdx.x; i < heads * pad; i += 256) {
+    // (blockIdx.y: with few rows several blocks share a row's outputs; each makes the row's statistics for itself)
+    const int first = threadIdx.x + 256 * blockIdx.y, stride = 256 * gridDim.y;
+    for (int i = first; i < heads * pad; i += stride) {
         const int h = i / pad, c = i % pad;
         store_f32(q_out + row * (size_t)(heads * pad) + i, c < dim ? turned(0, qw, h * dim, c, rq) : 0.f);
     }
@@ -184,7 +186,7 @@ whole_norm_rope_scatter_kernel(const float* __restrict__ proj, int ld, const flo
     const int slot = slots[row];
     if (slot < 0) return;
     const size_t page = slot / page_size, off = slot % page_size;
-    for (int i = threadIdx.x; i < kv_heads * pad; i += 256) {
+    for (int i = first; i < kv_heads * pad; i += stride) {
         const int h = i / pad, c = i % pad;
         const float kv = c < dim ? turned(nq, kw, h * dim, c, rk) : 0.f;
         const float vv = c < vdim ? val(nq + nk + h * vdim + c) * (value_norm ? rv[h] : 1.0f) : 0.f;
@@ -202,11 +204,12 @@ extern "C" int cisr_whole_norm_rope_scatter(const float* proj, int ld, const flo
     if (dim <= 0 || dim > pad || vdim > pad || 2 * half > dim || half < 0 || heads <= 0 || (has_kv && (kv_heads <= 0 || page_size <= 0)) ||
         (value_norm && kv_heads > WN_MAX_KV_HEADS))
         return (int)hipErrorInvalidValue;
+    const dim3 grid(rows, rows <= 128 ? 4 : 1);
     if (dtype == DT_F32)
-        whole_norm_rope_scatter_kernel<float><<<rows, 256, 0, stream>>>(proj, ld, bias, qw, kw, positions, slots, cosines, sines, half, max_pos,
+        whole_norm_rope_scatter_kernel<float><<<grid, 256, 0, stream>>>(proj, ld, bias, qw, kw, positions, slots, cosines, sines, half, max_pos,
             (float*)q_out, (float*)kcache, (float*)vcache, heads, kv_heads, dim, vdim, pad, page_size, eps, has_kv, split_half, value_norm);
     else
-        whole_norm_rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, ld, bias, qw, kw, positions, slots, cosines, sines, half, max_pos,
+        whole_norm_rope_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(proj, ld, bias, qw, kw, positions, slots, cosines, sines, half, max_pos,
             (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, vdim, pad, page_size, eps, has_kv, split_half, value_norm);
     return CISR_LAUNCH_CHECK();
 }
