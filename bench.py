@@ -433,7 +433,7 @@ def design_configs(width, layers, context):
     # feed-forwards alternate between dense (4 x width, squared relu, biases: 8 width^2) and 14 gated experts of width / 2
     # plus 2 identity experts in 4 groups of which 2 are kept, 4 chosen, and a shared expert of the width (9 width^2 active)
     talk = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
-            "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 4.0}}}
+            "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0}}}
     memory = {"heads": heads, "dim": 64, "vdim": 128, "gate_cap": 15.0}
     pair = {"left": talk, "right": memory, "left_scale": 1.0, "right_scale": 1.0}
     scored = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 14, "top": 4, "identity": 2, "groups": {"count": 4, "keep": 2}},
