@@ -67,7 +67,7 @@ def rounded(a, dtype):
     (4, 2, 24, 16, 20, None, 16, True, True), (1, 1, 10, 24, 1, None, 16, True, False), (20, 4, 64, 64, 100, None, 8, True, True),
     (3, 3, 16, 40, None, None, 16, False, True), (6, 2, 8, 8, None, 33, 4, True, False), (40, 8, 32, 48, 70, None, 16, True, True),
     (16, 4, 128, 128, 128, None, 16, True, True), (32, 8, 96, 80, None, None, 32, False, True), (10, 5, 112, 72, 64, None, 16, True, False),
-    (64, 16, 128, 64, 50, None, 16, True, True), (12, 12, 136, 160, 90, None, 16, True, True)])
+    (64, 16, 128, 64, 50, None, 16, True, True), (12, 12, 136, 160, 90, None, 16, True, True), (4, 2, 192, 256, 40, None, 16, True, True)])
 def test_attention_with_mixed_scores_alone(dtype, heads, kv_heads, dim, vdim, chunk, window, page_size, sink, gate):
     """Rows of three requests (a long portion, a single token far into its sequence, a sequence's first tokens) against
     the plain sums; the pages lie scattered, pages before a row's block are not there (-1 in the table).  One query and
@@ -629,3 +629,94 @@ def test_command_line_serves_the_design(folders, tmp_path):
     out = json.loads(proc.stdout)
     assert out["weights"] == "random-zovozen-tiny" and len(out["requests"][0]["generated"]) == 3
     assert out["runner"]["replays"] >= 1 and out["runner"]["cache"][0]["resident_pages"] == 0
+
+
+# -- configurations drawn at random -----------------------------------------------------------------------------------
+
+def random_config(seed):
+    """A configuration drawn at random: sizes, head counts, blocks of positions, rotation, constants, the kinds of
+    feed-forward in an order of their own.  Every second draw has sizes of the order of a small real model (heads of 64
+    to 128, a width of a few hundred, a dozen experts)."""
+    from zovozen_models import config, dense, layer, left, moe, right
+    rng = np.random.default_rng(1000 + seed)
+    pick = lambda *values: values[int(rng.integers(len(values)))]
+    big = seed % 2 == 1
+    width = pick(192, 264, 384) if big else pick(40, 72, 100, 136)
+
+    def feed_forward():
+        kind = rng.random()
+        if kind < 0.15:
+            return None
+        if kind < 0.4:
+            return dense(pick(256, 520) if big else pick(24, 60, 100))
+        count = pick(1, 2, 4)
+        per = pick(2, 3, 4) if big else pick(1, 2, 3)
+        outputs = count * per
+        identity = min(pick(0, 0, 1, 2), outputs - 1)
+        keep = int(rng.integers(1, count + 1))
+        top = int(rng.integers(1, min(keep * per, 6) + 1))
+        groups = None if count == 1 and rng.random() < 0.5 else (count, keep)
+        return moe(pick(48, 80, 136) if big else pick(8, 20, 33), outputs - identity, top, identity, groups, pick(None, 16, 40))
+
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        kv_heads = pick(1, 2, 3)
+        heads = kv_heads * pick(1, 2, 4)
+        dim = pick(64, 96, 128) if big else pick(6, 16, 24, 40)
+        vdim = pick(dim, 32, 64, 80, 128) if big else pick(dim, 8, 12, 48)
+        dims = pick(dim, dim // 2, 2, 4)
+        rot = pick(None, (float(pick(50.0, 10000.0, 1e6)), dims - dims % 2 or 2, pick(None, 2.0, 8.0)))
+        chunk = pick(None, 1, 2, 15, 16, 17, 33, 64, 90)
+        mem_heads = pick(1, 2, 4, 6)
+        layers.append(layer(left(heads, kv_heads, dim, vdim, float(rng.uniform(0.08, 0.4)), chunk, rot),
+                            right(mem_heads, pick(32, 64) if big else pick(4, 8, 20), pick(32, 64, 100) if big else pick(5, 8, 16, 24), float(rng.uniform(2.0, 20.0))),
+                            float(rng.uniform(0.3, 2.0)), float(rng.uniform(0.3, 2.0)), feed_forward()))
+    return config(int(rng.integers(40, 700)), width, pick(1e-5, 1e-6), layers)
+
+
+_DRAWN = {}
+
+
+@pytest.fixture(scope="module")
+def drawn(tmp_path_factory):
+    """seed -> (configuration, folder, trace, sequences), made once for both dtypes."""
+    def make(seed):
+        if seed not in _DRAWN:
+            cfg = random_config(seed)
+            folder = write_folder(tmp_path_factory.mktemp(f"drawn{seed}") / "model", cfg, 300 + seed, sharp=seed % 3 == 0)
+            lengths = (70, 33, 90, 9, 48) if seed % 2 else (70, 33, 120, 9, 64, 97)
+            trace, seqs = mixed(cfg["vocab"], seed=40 + seed, lengths=lengths)
+            _DRAWN[seed] = (cfg, folder, trace, seqs)
+        return _DRAWN[seed]
+    return make
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random_in_mixed_batches(drawn, tmp_path, seed, dtype):
+    """float32 holds its bound at every position but the few that the design itself magnifies (see
+    test_blocks_give_their_pages_back).  In bfloat16 a router's close call, or a memory's sign at a first position, may
+    fall otherwise than in float64 and reaches the positions after it through caches and states, so every position is
+    compared alone: the median holds half the bound and at most a quarter of the positions miss it."""
+    from runtime.engine.replay import replay
+    cfg, folder, trace, seqs = drawn(seed)
+    V = cfg["vocab"]
+    done = []
+    runner = replay(folder, dtype, tmp_path / "out", trace.peak, trace.lines(), echo=done.append, execution="graph" if seed % 2 else "eager")
+    assert done == [f"done {i}" for i in range(len(trace.steps))]
+    runner.cache.check()
+    errs = []
+    for step, rows in trace.expect.items():
+        data = np.fromfile(tmp_path / "out" / f"{step}.f32", dtype="<f4").reshape(len(rows), V).astype(np.float64)
+        for row, (rid, pos) in zip(data, rows):
+            want = plain_logits(folder, seqs[rid])[pos]
+            assert np.isfinite(row).all()
+            if dtype == "float32":
+                errs.append(np.abs(row - want).max() / np.abs(plain_logits(folder, seqs[rid])).max())
+            else:
+                errs.append(np.linalg.norm(row - want) / np.linalg.norm(want))
+    errs = np.sort(np.asarray(errs))
+    if dtype == "float32":
+        assert errs[-1] < 20 * conftest.F32_TOL and errs[:-3].max() < conftest.F32_TOL, f"float32: worst {errs[-4:]}"
+    else:
+        assert (errs > conftest.BF16_RMSE).mean() <= 0.25 and np.median(errs) < 0.5 * conftest.BF16_RMSE, f"bfloat16: median {np.median(errs):.3e}, worst {errs[-4:]}"
