@@ -67,7 +67,7 @@ def rounded(a, dtype):
     (4, 2, 24, 16, 20, None, 16, True, True), (1, 1, 10, 24, 1, None, 16, True, False), (20, 4, 64, 64, 100, None, 8, True, True),
     (3, 3, 16, 40, None, None, 16, False, True), (6, 2, 8, 8, None, 33, 4, True, False), (40, 8, 32, 48, 70, None, 16, True, True),
     (16, 4, 128, 128, 128, None, 16, True, True), (32, 8, 96, 80, None, None, 32, False, True), (10, 5, 112, 72, 64, None, 16, True, False),
-    (64, 16, 128, 64, 50, None, 16, True, True), (12, 12, 136, 160, 90, None, 16, True, True), (4, 2, 192, 256, 40, None, 16, True, True)])
+    (64, 16, 128, 64, 50, None, 16, True, True), (12, 12, 136, 160, 90, None, 16, True, True), (4, 2, 192, 256, 40, None, 16, True, True), (24, 8, 128, 120, 200, None, 16, True, True)])
 def test_attention_with_mixed_scores_alone(dtype, heads, kv_heads, dim, vdim, chunk, window, page_size, sink, gate):
     """Rows of three requests (a long portion, a single token far into its sequence, a sequence's first tokens) against
     the plain sums; the pages lie scattered, pages before a row's block are not there (-1 in the table).  One query and
